@@ -179,9 +179,14 @@ def require_positive(origin: str, **named: int) -> None:
 
 
 def architecture_name(data: Dict[str, Any], origin: str) -> str:
+    """The name a configuration is registered under: ``architectures[0]``, or the string ``architecture`` of a
+    config.json that has no such list."""
     archs = data.get("architectures")
+    if archs is None and isinstance(data.get("architecture"), str) and data["architecture"]:
+        return data["architecture"]
     if not isinstance(archs, Sequence) or isinstance(archs, str) or len(archs) == 0 or not isinstance(archs[0], str):
-        raise ConfigError(f"'{origin}': key 'architectures' must be a list that starts with the model's class name")
+        raise ConfigError(f"'{origin}': key 'architectures' must be a list that starts with the model's class name "
+                          f"(or 'architecture' a string)")
     return archs[0]
 
 

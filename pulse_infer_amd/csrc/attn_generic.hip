@@ -8,6 +8,9 @@
 // parameter (the reference fixes rsqrt(head_size), paged_attention.cu:108), and
 // query head h reads kv head h / (nq / nkv) (paged_attention.cu:61-70).
 //
+// With `gate` every head's output is multiplied by sigmoid(gate[token, head]) before it is stored (an output gate
+// whose logits another product left, one a token and head, `gate_stride` elements from row to row).
+//
 // This is the kernel of the true 32-bit path and the fallback for sizes that the
 // matrix-core kernels refuse.
 #include "common.h"
@@ -32,7 +35,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const TX* __restrict__
                                                           const TC* __restrict__ vcache,
                                                           const int* __restrict__ positions,
                                                           const int* __restrict__ token_entry,
-                                                          const int* __restrict__ block_table, AttnArgs a) {
+                                                          const int* __restrict__ block_table,
+                                                          const TX* __restrict__ gate, int64_t gate_stride, AttnArgs a) {
     extern __shared__ long long lds[];
     long long* v_s = lds;                                         // [64] value offsets of a tile's keys
     float* p_s = reinterpret_cast<float*>(lds + PULSE_WAVE);      // [64] a tile's probabilities
@@ -101,7 +105,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const TX* __restrict__
     }
 
     TX* orow = out + static_cast<int64_t>(t) * a.o_stride + static_cast<int64_t>(h) * d;
-    const float inv_l = l > 0.f ? 1.0f / l : 0.f;
+    float inv_l = l > 0.f ? 1.0f / l : 0.f;
+    if (gate) inv_l *= 1.0f / (1.0f + expf(-to_f32<TX>(gate[static_cast<int64_t>(t) * gate_stride + h])));
 #pragma unroll
     for (int r = 0; r < MAX_ACC; ++r) {
         const int e = lane + r * PULSE_WAVE;
@@ -115,7 +120,7 @@ extern "C" int pulse_attn_generic(const void* q, int64_t q_stride, void* out, in
                                   const void* kcache, const void* vcache, int c_dtype, const int* positions,
                                   const int* token_entry, const int* block_table, int bt_width, int tokens, int nq,
                                   int nkv, int d, int page_size, int num_pages, float scale, int window,
-                                  hipStream_t stream) {
+                                  const void* gate, int64_t gate_stride, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && nq > 0 && nkv > 0 && d > 0, "attn_generic: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_generic: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(d <= PULSE_WAVE * MAX_ACC, "attn_generic: head_dim %d exceeds %d", d, PULSE_WAVE * MAX_ACC);
@@ -126,6 +131,7 @@ extern "C" int pulse_attn_generic(const void* q, int64_t q_stride, void* out, in
                   "attn_generic: row strides too small");
     PULSE_REQUIRE(pulse_dtype_ok(x_dtype) && pulse_dtype_ok(c_dtype), "attn_generic: bad dtype tag");
     PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table, "attn_generic: null pointer");
+    PULSE_REQUIRE(!gate || gate_stride >= nq, "attn_generic: the gate's rows are too short");
     if (tokens == 0) return 0;
     AttnArgs a;
     a.nq = nq; a.nkv = nkv; a.d = d; a.q_stride = q_stride; a.o_stride = o_stride;
@@ -134,7 +140,8 @@ extern "C" int pulse_attn_generic(const void* q, int64_t q_stride, void* out, in
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(c_dtype, TC,
         hipLaunchKernelGGL((attn_generic_kernel<TX, TC>), dim3(tokens, nq), dim3(64), lds, stream,
                            static_cast<const TX*>(q), static_cast<TX*>(out), static_cast<const TC*>(kcache),
-                           static_cast<const TC*>(vcache), positions, token_entry, block_table, a)));
+                           static_cast<const TC*>(vcache), positions, token_entry, block_table,
+                           static_cast<const TX*>(gate), gate_stride, a)));
     PULSE_LAUNCH_CHECK("attn_generic");
     return 0;
 }

@@ -43,13 +43,14 @@ extern "C" int pulse_embed_gather(const int* ids, const void* table, int table_d
 // For output row r (input row s = rows ? rows[r] : r):
 //   v = h[s] + delta[s]            (delta optional)
 //   h[s] = v                       (only when write_back)
-//   y[r] = v * (1 / sqrt(mean(v^2) + eps)) * w      one rounding at the end
+//   y[r] = v * (1 / sqrt(mean(v^2) + eps)) * (w_offset + w)      one rounding at the end
+// (w_offset: 0 for a weight stored as the factor itself, 1 for a weight stored as the factor's distance from one)
 // (formula: src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157; the reference adds the
 // residual in a separate kernel, src/ops/kernels/cuda/add_kernel.cu:73-92)
 template <typename TD, typename TW, typename TY>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int parts, int64_t part_stride,
                                    const int* __restrict__ rows, const TW* __restrict__ w,
-                                   TY* __restrict__ y, int hidden, float eps, int write_back) {
+                                   TY* __restrict__ y, int hidden, float eps, int write_back, float w_offset) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int64_t s = rows ? rows[r] : r;
@@ -70,7 +71,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
         if (drow)
             for (int p = 0; p < parts; ++p) v += to_f32<TD>(drow[p * part_stride + i]);
         if (write_back) hrow[i] = v;
-        yrow[i] = from_f32<TY>(v * inv * to_f32<TW>(w[i]));
+        yrow[i] = from_f32<TY>(v * inv * (w_offset + to_f32<TW>(w[i])));
     }
 }
 
@@ -99,7 +100,7 @@ template <typename TD, typename TW, typename TY, int THREADS, bool PARTS>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               int parts, int64_t part_stride,
                                                               const int* __restrict__ rows, const TW* __restrict__ w,
-                                                              TY* __restrict__ y, int hidden, float eps, int write_back) {
+                                                              TY* __restrict__ y, int hidden, float eps, int write_back, float w_offset) {
     __shared__ float scratch[16];
     typedef typename Vec4<TD>::type VD;
     typedef typename Vec4<TW>::type VW;
@@ -162,7 +163,8 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
         const int i = threadIdx.x + c * THREADS;
         if (i < nvec) {
             if (write_back) hrow[i] = v[c];
-            const float4 ww = widen4(wv[i]);
+            float4 ww = widen4(wv[i]);
+            ww.x += w_offset; ww.y += w_offset; ww.z += w_offset; ww.w += w_offset;
             yrow[i] = narrow4<TY>(make_float4(v[c].x * inv * ww.x, v[c].y * inv * ww.y, v[c].z * inv * ww.z,
                                               v[c].w * inv * ww.w));
         }
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
 // order, is what is normalised (the shares of a product whose inner dimension was split).
 extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, int parts, int64_t part_stride,
                                  const int* rows, const void* w, int w_dtype, void* y, int y_dtype, int out_rows,
-                                 int hidden, float eps, int write_back, hipStream_t stream) {
+                                 int hidden, float eps, int write_back, float w_offset, hipStream_t stream) {
     PULSE_REQUIRE(parts >= 1 && (parts == 1 || (delta && part_stride % 4 == 0)), "add_rmsnorm: bad parts of the update");
     PULSE_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
     PULSE_REQUIRE(pulse_dtype_ok(delta_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(y_dtype),
@@ -188,20 +190,20 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, i
             if (parts > 1)
                 hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024, true>), dim3(out_rows), dim3(1024), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                                   static_cast<TY*>(y), hidden, eps, write_back);
+                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset);
             else if (out_rows <= 256 && hidden >= 2048)   // few rows: bound by round trips, not by bandwidth
                 hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024, false>), dim3(out_rows), dim3(1024), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                                   static_cast<TY*>(y), hidden, eps, write_back);
+                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset);
             else
                 hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 256, false>), dim3(out_rows), dim3(256), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                                   static_cast<TY*>(y), hidden, eps, write_back))));
+                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset))));
     } else {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
             hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
                                static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                               static_cast<TY*>(y), hidden, eps, write_back))));
+                               static_cast<TY*>(y), hidden, eps, write_back, w_offset))));
     }
     PULSE_LAUNCH_CHECK("add_rmsnorm");
     return 0;

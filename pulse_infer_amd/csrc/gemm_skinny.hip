@@ -71,7 +71,8 @@ template <int SLABS, int MT, int KW, bool SWIGLU>
 __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void* __restrict__ C, int64_t ldc, int M, int N,
                                          int n_base, int mode, int tid, float* __restrict__ sumsq = nullptr, int parts = 0,
                                          const float* row_scale = nullptr, bf16_t* __restrict__ copy = nullptr,
-                                         int64_t ldcopy = 0, const bf16_t* __restrict__ copy_scale = nullptr) {
+                                         int64_t ldcopy = 0, const bf16_t* __restrict__ copy_scale = nullptr,
+                                         float copy_offset = 0.f) {
     constexpr int TILES = SLABS * MT;
     constexpr int THREADS = KW * PULSE_WAVE;
     if (!SWIGLU) {
@@ -95,7 +96,7 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
                     static_cast<float*>(C)[at] = updated;
                     if (copy)
                         copy[static_cast<int64_t>(m) * ldcopy + n] =
-                            f32_to_bf16(copy_scale ? updated * bf16_to_f32(copy_scale[n]) : updated);
+                            f32_to_bf16(copy_scale ? updated * (copy_offset + bf16_to_f32(copy_scale[n])) : updated);
                 }
             }
             if (sumsq) {  // the 16 lanes of a row of lanes hold the 16 columns of one row of the tile
@@ -291,7 +292,8 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                                                                              int N, int K, int mode, RowScale scale,
                                                                              float* __restrict__ sumsq_out, int parts_out,
                                                                              bf16_t* __restrict__ copy_out, int64_t ldcopy,
-                                                                             const bf16_t* __restrict__ copy_scale) {
+                                                                             const bf16_t* __restrict__ copy_scale,
+                                                                             float copy_offset) {
     constexpr int THREADS = KW * PULSE_WAVE;
     static_assert(PACK == 1 || PACK == 2 || PACK == 4 || PACK == 8, "PACK k-steps a load of X");
     static_assert(UNROLL % 2 == 0 && UNROLL % PACK == 0, "groups hold whole pairs and whole packs");
@@ -438,7 +440,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
         for (int i = 0; i < 4; ++i) red[wave][s][4 * kg + i][r] = acc[s][i];
     __syncthreads();
     epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid, sumsq_out, parts_out,
-                                   SCALED ? s_rstd : nullptr, copy_out, ldcopy, copy_scale);
+                                   SCALED ? s_rstd : nullptr, copy_out, ldcopy, copy_scale, copy_offset);
 }
 
 template <int SLABS, int MT, int KW, bool SWIGLU>
@@ -460,12 +462,12 @@ void launch(bool xlds, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ld
 template <int SLABS, int KW, bool SWIGLU>
 void launch_stream(int pack, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                    int K, int mode, const RowScale& scale, float* sumsq_out, int parts_out, bf16_t* copy_out, int64_t ldcopy,
-                   const bf16_t* copy_scale, hipStream_t stream) {
+                   const bf16_t* copy_scale, float copy_offset, hipStream_t stream) {
     const dim3 grid((N + SLABS * 16 - 1) / (SLABS * 16)), block(KW * PULSE_WAVE);
     const size_t red_bytes = sizeof(float) * KW * SLABS * 16 * 17;
 #define PULSE_STREAM(P, SCALED)                                                                                          \
     hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU, SCALED>), grid, block, red_bytes, stream, X, ldx, \
-                       W, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy_out, ldcopy, copy_scale)
+                       W, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy_out, ldcopy, copy_scale, copy_offset)
 #define PULSE_STREAM_PACKS(SCALED)                    \
     do {                                              \
         if (pack == 8) PULSE_STREAM(8, SCALED);       \
@@ -495,14 +497,15 @@ int pack_for(int M) { return M <= 2 ? 8 : (M <= 4 ? 4 : (M <= 8 ? 2 : 1)); }
 //   sumsq_out != null (mode 2 only): besides adding into C, leave sumsq_out[row * parts + slab] = sum of squares of the
 //     new values of C[row, 16 slab .. 16 slab + 15], parts = ceil(N / 16);
 //   copy_out != null (mode 2 only): the new values of C once more as bfloat16, row stride ldcopy, each multiplied by
-//     copy_scale[column] first (bfloat16 [N], the weight of the norm that reads C next; null: as they are).
+//     copy_offset + copy_scale[column] first (bfloat16 [N], the weight of the norm that reads C next, and what that
+//     norm adds to its weight: 0, or 1 for a weight stored as its distance from one; null: as they are).
 // pulse_gemm_skinny_fusable says whether the streaming kernel takes a shape.
 extern "C" int pulse_gemm_skinny_fusable(int M, int N, int K) { return M >= 1 && M <= 16 && N > 0 && K > 0 && K % 1024 == 0; }
 
 extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
                                        int N, int K, int mode, int swiglu, int tune, const float* scale_sumsq,
                                        int scale_parts, float scale_eps, float* sumsq_out, void* copy_out,
-                                       int64_t ldcopy, const void* copy_scale, hipStream_t stream) {
+                                       int64_t ldcopy, const void* copy_scale, float copy_offset, hipStream_t stream) {
     const bool fused = scale_sumsq != nullptr || sumsq_out != nullptr || copy_out != nullptr;
     if (fused) {
         PULSE_REQUIRE(pulse_gemm_skinny_fusable(M, N, K) && tune != 9, "gemm_skinny: M=%d N=%d K=%d cannot take the fused kernel", M, N, K);
@@ -556,14 +559,14 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
         const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
         const int pack = t_pack ? t_pack : pack_for(M);
         if (swiglu) {
-            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
-            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
+            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, copy_offset, stream);
+            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, copy_offset, stream);
         } else if (slabs == 2) {
-            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
-            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
+            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, copy_offset, stream);
+            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, copy_offset, stream);
         } else {
-            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
-            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
+            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, copy_offset, stream);
+            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, copy_offset, stream);
         }
         PULSE_LAUNCH_CHECK("gemm_skinny");
         return 0;
@@ -590,5 +593,5 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
 extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
                                  int N, int K, int mode, int swiglu, int tune, hipStream_t stream) {
     return pulse_gemm_skinny_fused(X, ldx, W, ldw, C, ldc, M, N, K, mode, swiglu, tune, nullptr, 0, 0.f, nullptr, nullptr, 0,
-                                   nullptr, stream);
+                                   nullptr, 0.f, stream);
 }

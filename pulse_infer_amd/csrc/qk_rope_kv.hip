@@ -10,6 +10,11 @@
 // page write: src/model/qwen3/model.cpp:815-848; formulas
 // src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157, rope_kernel.cu:76-132,
 // paged_kv_write.cu:31-52).  Norm and rotation are float32 with one rounding.
+//
+// Options beyond that: the norm may have no weights (a division by the head's root mean square alone); q may be
+// multiplied by a temperature that grows with the position, 1 + coef * ln(floor((pos + 1) / every) + 1), in float32
+// after the norm; and the values may be taken from any head-sized columns of the row (`v_head0`: the head number at
+// which they start), e.g. from the raw key columns for a design whose values are its keys as projected.
 #include "common.h"
 
 namespace {
@@ -24,7 +29,17 @@ struct QkRopeArgs {
     int pairing;     // 0: (2i, 2i+1)   1: (i, i + rotary_dim/2)
     int page_size, num_pages, bt_width;
     int write_kv;
+    int norm;        // 0: none   1: with the weights q_w / k_w   2: without weights
+    int v_head0;     // the values of kv head g are columns (v_head0 + g) * d .. of the row
+    float temp_coef; // query temperature: q *= 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1); temp_every 0: none
+    int temp_every;
 };
+
+// The factor of the query temperature at a position (1 when there is none).
+__device__ __forceinline__ float query_temperature(const QkRopeArgs& a, int pos) {
+    if (a.temp_every <= 0) return 1.f;
+    return 1.f + a.temp_coef * logf(static_cast<float>((pos + 1) / a.temp_every) + 1.f);
+}
 
 template <typename TX, typename TW, typename TC>
 __global__ __launch_bounds__(64) void qk_rope_kv_kernel(TX* __restrict__ qkv, const TW* __restrict__ q_w,
@@ -80,10 +95,11 @@ __global__ __launch_bounds__(64) void qk_rope_kv_kernel(TX* __restrict__ qkv, co
     }
     float vv[2 * MAX_PAIRS_PER_LANE];
     int pos = 0, entry = 0;
+    if (is_q && a.temp_every > 0) pos = positions[t];
     if (!is_q) {
         pos = positions[t];
         entry = token_entry[t];
-        const TX* v = row + static_cast<int64_t>(a.nq + a.nkv + g) * d;
+        const TX* v = row + static_cast<int64_t>(a.v_head0 + g) * d;
 #pragma unroll
         for (int r = 0; r < 2 * MAX_PAIRS_PER_LANE; ++r) {
             const int i = lane + r * PULSE_WAVE;
@@ -104,22 +120,27 @@ __global__ __launch_bounds__(64) void qk_rope_kv_kernel(TX* __restrict__ qkv, co
     }
 
     float inv = 1.f;
-    if (w) {
+    if (a.norm) {
         float ss = 0.f;
 #pragma unroll
         for (int r = 0; r < MAX_PAIRS_PER_LANE; ++r) ss += xa[r] * xa[r] + xb[r] * xb[r];
         ss = wave_sum(ss);
         inv = 1.0f / sqrtf(ss / static_cast<float>(d) + a.eps);
     }
+    const float temp = is_q ? query_temperature(a, pos) : 1.f;
 
 #pragma unroll
     for (int r = 0; r < MAX_PAIRS_PER_LANE; ++r) {
         const int p = lane + r * PULSE_WAVE;
         if (p < npairs) {
             float va = xa[r], vb = xb[r];
-            if (w) {
+            if (a.norm) {
                 va = va * inv * wa[r];
                 vb = vb * inv * wb[r];
+            }
+            if (a.temp_every > 0) {
+                va *= temp;
+                vb *= temp;
             }
             if (p < half_rot && cos_t) {
                 const float ra = va * cs[r] - vb * sn[r];
@@ -257,6 +278,7 @@ __global__ __launch_bounds__(64) void qk_rope_kv_vec_kernel(bf16_t* __restrict__
     }
     const bool is_k = on && !is_q;
     int pos = 0, entry = 0;
+    if (a.temp_every > 0) pos = positions[t];
     if (is_k) {
         pos = positions[t];
         entry = token_entry[t];
@@ -276,7 +298,7 @@ __global__ __launch_bounds__(64) void qk_rope_kv_vec_kernel(bf16_t* __restrict__
         for (int i = 0; i < 8; ++i) e[i] = 0.f;
     }
     float inv = 1.f;
-    if (w) {
+    if (a.norm) {
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) ss += e[i] * e[i];
@@ -285,6 +307,11 @@ __global__ __launch_bounds__(64) void qk_rope_kv_vec_kernel(bf16_t* __restrict__
         inv = 1.0f / sqrtf(ss / static_cast<float>(d) + a.eps);
 #pragma unroll
         for (int i = 0; i < 8; ++i) e[i] = e[i] * inv * wv[i];
+    }
+    if (a.temp_every > 0 && is_q) {
+        const float temp = query_temperature(a, pos);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] *= temp;
     }
     if (rotated) {
 #pragma unroll
@@ -330,7 +357,7 @@ __global__ __launch_bounds__(VW_THREADS) void v_page_write_kernel(const bf16_t* 
     const int page = block_table[static_cast<int64_t>(token_entry[t]) * a.bt_width + pos / a.page_size];
     if (page < 0 || page >= a.num_pages) return;
     const int slot = pos % a.page_size;
-    const bf16_t* src = qkv + static_cast<int64_t>(t) * a.row_stride + static_cast<int64_t>(a.nq + a.nkv + g) * a.d;
+    const bf16_t* src = qkv + static_cast<int64_t>(t) * a.row_stride + static_cast<int64_t>(a.v_head0 + g) * a.d;
     bf16_t* dst = vcache + (static_cast<int64_t>(page) * a.nkv + g) * a.d * a.page_size + slot;
     for (int c0 = cg * 8; c0 < a.d; c0 += 8 * (VW_THREADS / VW_TOKENS)) {
         const uint4 raw = *reinterpret_cast<const uint4*>(src + c0);
@@ -363,7 +390,8 @@ extern "C" int pulse_qk_rope_kv(void* qkv, int x_dtype, int64_t row_stride, cons
                                 int w_dtype, float eps, const float* cos_t, const float* sin_t, int rotary_dim,
                                 int pairing, void* kcache, void* vcache, int c_dtype, const int* positions,
                                 const int* token_entry, const int* block_table, int bt_width, int tokens, int nq,
-                                int nkv, int d, int page_size, int num_pages, int write_kv, hipStream_t stream) {
+                                int nkv, int d, int page_size, int num_pages, int write_kv, int plain_norm,
+                                int v_head0, float temp_coef, int temp_every, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && nq > 0 && nkv >= 0 && d > 0, "qk_rope_kv: bad sizes");
     PULSE_REQUIRE(d % 2 == 0 && d <= 2 * PULSE_WAVE * MAX_PAIRS_PER_LANE,
                   "qk_rope_kv: head_dim %d must be even and at most %d", d, 2 * PULSE_WAVE * MAX_PAIRS_PER_LANE);
@@ -371,13 +399,16 @@ extern "C" int pulse_qk_rope_kv(void* qkv, int x_dtype, int64_t row_stride, cons
                   "qk_rope_kv: rotary_dim %d must be even and at most head_dim %d", rotary_dim, d);
     PULSE_REQUIRE(pairing == 0 || pairing == 1, "qk_rope_kv: unknown pairing %d", pairing);
     PULSE_REQUIRE((q_w == nullptr) == (k_w == nullptr), "qk_rope_kv: give both norm weights or neither");
+    PULSE_REQUIRE(!(plain_norm && q_w), "qk_rope_kv: a norm without weights was asked for and weights were given");
+    PULSE_REQUIRE(temp_every >= 0, "qk_rope_kv: the query temperature's interval must not be negative");
     PULSE_REQUIRE(rotary_dim == 0 || (cos_t && sin_t), "qk_rope_kv: rotation needs the cos/sin tables");
     PULSE_REQUIRE(pulse_dtype_ok(x_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(c_dtype), "qk_rope_kv: bad dtype tag");
     PULSE_REQUIRE(qkv && positions, "qk_rope_kv: null pointer");
     if (write_kv) {
         PULSE_REQUIRE(kcache && vcache && token_entry && block_table, "qk_rope_kv: cache pointers missing");
         PULSE_REQUIRE(page_size > 0 && num_pages > 0 && bt_width > 0 && nkv > 0, "qk_rope_kv: bad cache geometry");
-        PULSE_REQUIRE(row_stride >= static_cast<int64_t>(nq + 2 * nkv) * d, "qk_rope_kv: row stride too small");
+        PULSE_REQUIRE(v_head0 >= 0 && row_stride >= static_cast<int64_t>(nq + nkv) * d &&
+                      row_stride >= static_cast<int64_t>(v_head0 + nkv) * d, "qk_rope_kv: row stride too small");
     } else {
         PULSE_REQUIRE(row_stride >= static_cast<int64_t>(nq) * d, "qk_rope_kv: row stride too small");
     }
@@ -386,6 +417,7 @@ extern "C" int pulse_qk_rope_kv(void* qkv, int x_dtype, int64_t row_stride, cons
     a.nq = nq; a.nkv = nkv; a.d = d; a.row_stride = row_stride; a.eps = eps;
     a.rotary_dim = (cos_t ? rotary_dim : 0); a.pairing = pairing;
     a.page_size = page_size; a.num_pages = num_pages; a.bt_width = bt_width; a.write_kv = write_kv;
+    a.norm = q_w ? 1 : (plain_norm ? 2 : 0); a.v_head0 = v_head0; a.temp_coef = temp_coef; a.temp_every = temp_every;
     const int heads = write_kv ? nq + nkv : nq;
     // the 16-byte path: bfloat16 activations and cache, 8-element chunks that the rotation does not cut
     const bool vec = x_dtype == PULSE_BF16 && (!write_kv || c_dtype == PULSE_BF16) && d % 8 == 0 && a.rotary_dim % 8 == 0 && row_stride % 8 == 0 &&

@@ -106,7 +106,32 @@ struct MfmaArgs {
     int rotary_dim;        // multiple of 8
     int pairing;           // 0: (2i, 2i+1)   1: (i, i + rotary_dim / 2), rotary_dim a multiple of 64
     int new_key;           // 1: the token's key and value are prepared, used and written to their page here
+    int plain_norm;        // 1: q and the key are divided by their root mean square although there are no norm weights
+    int v_head0;           // the token's raw value of kv head g: columns (v_head0 + g) D .. of its row (nq + nkv for a
+                           // projection of its own; nq for values that are the keys as projected)
+    float temp_coef;       // query temperature: q *= 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1), after the
+    int temp_every;        // norm; temp_every 0: none
+    // Every kernel that writes the output: head h of row t is multiplied by sigmoid(gate[t * gate_stride + h]) as it
+    // is stored (an output gate whose logits another product left); null: no gate.
+    const bf16_t* gate;
+    int64_t gate_stride;
 };
+
+// What the C entry points take besides their long lists (null: none of it).
+struct PulseAttnExtras {
+    const void* gate;      // bfloat16 [tokens, >= nq], row stride gate_stride
+    int64_t gate_stride;
+    int plain_norm;        // pulse_attn_decode only, as are the three below
+    int v_head0;           // < 0: nq + nkv
+    float temp_coef;
+    int temp_every;
+};
+
+// 1 / l of a column and its head's gate in one factor.
+__device__ __forceinline__ float gated(float inv, const bf16_t* gate, int64_t gate_stride, int64_t row, int head) {
+    if (!gate) return inv;
+    return inv / (1.0f + expf(-bf16_to_f32(gate[row * gate_stride + head])));
+}
 
 // The split size for a step whose longest context is `live` (at most n_splits * split_size, what the launch was made
 // for): the keys cut evenly into the launch's number of splits, in whole 32-key blocks, never more than split_size.
@@ -166,7 +191,8 @@ __device__ __forceinline__ void rotate_halves(float (&f)[NCHUNK][8], const HeadT
 // Per-head RMSNorm and rotation of one head whose 8-element slices ch*32 + kg*8.. sit in the four lanes kg = 0..3
 // of a column, with the arithmetic of qk_rope_kv.hip: float32, (x * inv) * w, then the rotation, one rounding.
 __device__ __forceinline__ void prepare_head(bf16x8 (&x)[NCHUNK], const HeadTables& tb, bool normed, bool rotated,
-                                             float eps, int rot, int pairing, int kg) {
+                                             float eps, int rot, int pairing, int kg, bool weighted = true,
+                                             float factor = 1.f) {
     float f[NCHUNK][8];
     float ss = 0.f;
 #pragma unroll
@@ -183,7 +209,14 @@ __device__ __forceinline__ void prepare_head(bf16x8 (&x)[NCHUNK], const HeadTabl
 #pragma unroll
         for (int ch = 0; ch < NCHUNK; ++ch)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) f[ch][e] = f[ch][e] * inv * static_cast<float>(tb.w[ch][e]);
+            for (int e = 0; e < 8; ++e)
+                f[ch][e] = weighted ? f[ch][e] * inv * static_cast<float>(tb.w[ch][e]) : f[ch][e] * inv;
+    }
+    if (factor != 1.f) {
+#pragma unroll
+        for (int ch = 0; ch < NCHUNK; ++ch)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[ch][e] *= factor;
     }
     if (rotated) {
         if (pairing == 0) {
@@ -301,7 +334,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
             const int half = a.rotary_dim / 2;
             const float* cos_row = a.cos_t ? a.cos_t + static_cast<int64_t>(row0) * half : nullptr;
             const float* sin_row = a.sin_t ? a.sin_t + static_cast<int64_t>(row0) * half : nullptr;
-            const bf16_t* vraw = a.q + static_cast<int64_t>(row0) * a.q_stride + static_cast<int64_t>(a.nq + a.nkv + g) * D;
+            const bf16_t* vraw = a.q + static_cast<int64_t>(row0) * a.q_stride + static_cast<int64_t>(a.v_head0 + g) * D;
 #pragma unroll
             for (int i = 0; i < VPL; ++i) vown[i] = (a.new_key && lane + i * PULSE_WAVE < D) ? vraw[lane + i * PULSE_WAVE] : 0;
 #pragma unroll
@@ -336,7 +369,10 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     u32x4* stash_k = s_newk[FUSED ? wave : 0];
     bf16_t* stash_v = s_newv[FUSED ? wave : 0];
     auto prepare = [&](bool own_key) {
-        prepare_head(bq, tb, a.q_w != nullptr, a.cos_t != nullptr, a.eps, a.rotary_dim, a.pairing, kg);
+        const float temp = a.temp_every > 0
+            ? 1.f + a.temp_coef * logf(static_cast<float>((max(pos_c, 0) + 1) / a.temp_every) + 1.f) : 1.f;
+        prepare_head(bq, tb, a.q_w != nullptr || a.plain_norm, a.cos_t != nullptr, a.eps, a.rotary_dim, a.pairing, kg,
+                     a.q_w != nullptr, temp);
         if (!col_ok) {
 #pragma unroll
             for (int ch = 0; ch < NCHUNK; ++ch) bq[ch] = zero8();
@@ -345,7 +381,8 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         // the key's norm weight takes the place of q's; cos and sin are the token's for both
 #pragma unroll
         for (int ch = 0; ch < NCHUNK; ++ch) tb.w[ch] = kwt[ch];
-        prepare_head(knew, tb, a.k_w != nullptr, a.cos_t != nullptr, a.eps, a.rotary_dim, a.pairing, kg);
+        prepare_head(knew, tb, a.k_w != nullptr || a.plain_norm, a.cos_t != nullptr, a.eps, a.rotary_dim, a.pairing, kg,
+                     a.k_w != nullptr);
         if (r == 0) {
 #pragma unroll
             for (int ch = 0; ch < NCHUNK; ++ch) {
@@ -599,7 +636,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int64_t row = row0 + tc2;
     const int head = g * a.group + hc2;
     if (a.n_splits == 1 || (a.plan && hi < split_size)) {   // the only split of its item: nothing to merge
-        const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+        const float inv = gated(ll > 0.f ? 1.0f / ll : 0.f, a.gate, a.gate_stride, row, head);
         bf16_t* dst = a.out + row * a.o_stride + static_cast<int64_t>(head) * D;
         for (int ch = dd; ch < D; ch += 16) {
             float v = 0.f;
@@ -856,7 +893,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     l_part += __shfl_xor(l_part, 16, PULSE_WAVE);
     l_part += __shfl_xor(l_part, 32, PULSE_WAVE);
     if (col_ok) {
-        const float inv = l_part > 0.f ? 1.0f / l_part : 0.f;
+        const float inv = gated(l_part > 0.f ? 1.0f / l_part : 0.f, a.gate, a.gate_stride, col_row, col_head);
         bf16_t* dst = a.out + static_cast<int64_t>(col_row) * a.o_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
@@ -1243,7 +1280,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
         l += __shfl_xor(l, 16, PULSE_WAVE);
         l += __shfl_xor(l, 32, PULSE_WAVE);
         if (col_ok[ct] && direct) {
-            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            const float inv = gated(l > 0.f ? 1.0f / l : 0.f, a.gate, a.gate_stride, col_row[ct], col_head);
             bf16_t* dst = a.out + static_cast<int64_t>(col_row[ct]) * a.o_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) {
@@ -1279,7 +1316,8 @@ __global__ __launch_bounds__(PR_THREADS) void attn_prefill_reduce_kernel(const f
                                                                         const int* __restrict__ positions,
                                                                         const int* __restrict__ items, int item_tokens,
                                                                         bf16_t* __restrict__ out, int64_t o_stride, int nq,
-                                                                        int n_splits, int split_size) {
+                                                                        int n_splits, int split_size,
+                                                                        const bf16_t* __restrict__ gate, int64_t gate_stride) {
     const int item = blockIdx.x / item_tokens;
     const int tok = blockIdx.x % item_tokens;
     const int row0 = items[4 * item];
@@ -1303,7 +1341,7 @@ __global__ __launch_bounds__(PR_THREADS) void attn_prefill_reduce_kernel(const f
         // a split below the row's window holds sums of nothing (zeros), never stale memory: it was written
         acc += *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad) * wz;
     }
-    const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+    const float inv = gated(ll > 0.f ? 1.0f / ll : 0.f, gate, gate_stride, row, head);
     const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[0] * inv)) | (static_cast<uint32_t>(f32_to_bf16(acc[1] * inv)) << 16);
     const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[2] * inv)) | (static_cast<uint32_t>(f32_to_bf16(acc[3] * inv)) << 16);
     *reinterpret_cast<u32x2*>(out + row * o_stride + static_cast<int64_t>(head) * D + 4 * quad) = u32x2{w0, w1};
@@ -1329,7 +1367,8 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
                                                                          bf16_t* __restrict__ out, int64_t o_stride, int nq,
                                                                          int n_splits, int static_split_size, int hpw_log2,
                                                                          const int* __restrict__ live_context,
-                                                                         const int* __restrict__ plan, int n_items) {
+                                                                         const int* __restrict__ plan, int n_items,
+                                                                         const bf16_t* __restrict__ gate, int64_t gate_stride) {
     __shared__ float s_w[MAX_SPLITS];      // hpw * n_splits <= MAX_SPLITS (hpw > 1 only with few splits)
     __shared__ float s_l[MAX_SPLITS];
     __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
@@ -1397,7 +1436,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
         for (int z = 0; z < valid; ++z) mm = fmaxf(mm, my_w[z]);
         float ll = 0.f;
         for (int z = 0; z < valid; ++z) ll += (my_w[z] == -INFINITY ? 0.f : exp2f(my_w[z] - mm)) * my_l[z];
-        inv = ll > 0.f ? 1.0f / ll : 0.f;
+        inv = gated(ll > 0.f ? 1.0f / ll : 0.f, gate, gate_stride, row, head);
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i) {
@@ -1549,11 +1588,23 @@ struct Preparation {
     int rotary_dim, pairing, new_key;
 };
 
+// The gate of `ex` into the kernels' arguments, checked; the other extras are pulse_attn_decode's.
+int take_gate(MfmaArgs& a, const PulseAttnExtras* ex, int nq) {
+    a.gate = nullptr; a.gate_stride = 0;
+    a.plain_norm = 0; a.v_head0 = a.nq + a.nkv; a.temp_coef = 0.f; a.temp_every = 0;
+    if (!ex || !ex->gate) return 0;
+    PULSE_REQUIRE(ex->gate_stride >= nq, "attention: the gate's rows hold %lld values for %d heads",
+                  static_cast<long long>(ex->gate_stride), nq);
+    a.gate = static_cast<const bf16_t*>(ex->gate); a.gate_stride = ex->gate_stride;
+    return 0;
+}
+
 int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
                      const void* vcache, const int* positions, const int* block_table, int bt_width, const int* items,
                      int n_items, int tokens, int nq, int nkv, int page_size, int num_pages, float scale, int window,
                      int split_size, int n_splits, int max_context, float* part_o, float* part_ml,
-                     const Preparation* prep, const int* live_context, const int* plan, hipStream_t stream) {
+                     const Preparation* prep, const int* live_context, const int* plan, const PulseAttnExtras* ex,
+                     hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_mfma: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_mfma: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page size %d must be a multiple of 16", page_size);
@@ -1591,6 +1642,16 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     a.plan = n_splits > 1 ? plan : nullptr;
     a.n_items = n_items;
     a.q_w = a.k_w = nullptr; a.cos_t = a.sin_t = nullptr; a.eps = 0.f; a.rotary_dim = 0; a.pairing = 0; a.new_key = 0;
+    if (take_gate(a, ex, nq)) return 1;
+    if (prep && ex) {
+        a.plain_norm = ex->plain_norm ? 1 : 0;
+        a.v_head0 = ex->v_head0 >= 0 ? ex->v_head0 : nq + nkv;
+        a.temp_coef = ex->temp_coef; a.temp_every = ex->temp_every;
+        PULSE_REQUIRE(!(a.plain_norm && (prep->q_w || prep->k_w)), "attn_decode: a norm without weights and weights at once");
+        PULSE_REQUIRE(a.temp_every >= 0, "attn_decode: the query temperature's interval must not be negative");
+        PULSE_REQUIRE(!prep->new_key || q_stride >= static_cast<int64_t>(a.v_head0 + nkv) * D,
+                      "attn_decode: the projection output's rows do not hold the values");
+    }
     if (prep) {
         a.q_w = static_cast<const bf16_t*>(prep->q_w); a.k_w = static_cast<const bf16_t*>(prep->k_w);
         a.cos_t = prep->cos_t; a.sin_t = prep->sin_t; a.eps = prep->eps; a.rotary_dim = prep->rotary_dim;
@@ -1608,7 +1669,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
         while (hpw * 2 * n_splits <= REDUCE_GROUPS && hpw * 2 <= nq) { hpw *= 2; ++hpw_log2; }
         hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, (nq + hpw - 1) / hpw), dim3(REDUCE_THREADS), 0, stream,
                            part_o, part_ml, positions, items, per, a.out, o_stride, nq, n_splits, split_size, hpw_log2,
-                           a.live_context, a.plan, n_items);
+                           a.live_context, a.plan, n_items, a.gate, a.gate_stride);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
     return 0;
@@ -1627,10 +1688,10 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
                                const int* items, int n_items, int tokens, int nq,
                                int nkv, int page_size, int num_pages, float scale, int window, int split_size,
                                int n_splits, int max_context, float* part_o, float* part_ml, const int* live_context,
-                               const int* plan, hipStream_t stream) {
+                               const int* plan, const PulseAttnExtras* extras, hipStream_t stream) {
     return launch_attn_mfma(q, q_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items, n_items,
                             tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits, max_context,
-                            part_o, part_ml, nullptr, live_context, plan, stream);
+                            part_o, part_ml, nullptr, live_context, plan, extras, stream);
 }
 
 // The plan of a step (see attn_plan_kernel) for pulse_attn_mfma / pulse_attn_decode with the same items and n_splits:
@@ -1670,7 +1731,8 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
                                  int num_pages, float scale, int window, int split_size, int n_splits, int max_context,
                                  float* part_o, float* part_ml, const void* q_w, const void* k_w, float eps,
                                  const float* cos_t, const float* sin_t, int rotary_dim, int pairing, int new_key,
-                                 const int* live_context, const int* plan, hipStream_t stream) {
+                                 const int* live_context, const int* plan, const PulseAttnExtras* extras,
+                                 hipStream_t stream) {
     PULSE_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin come together");
     if (!cos_t) rotary_dim = 0;
     PULSE_REQUIRE(pulse_attn_decode_takes(rotary_dim, pairing), "attn_decode: rotation of %d channels with pairing %d is not "
@@ -1678,13 +1740,14 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
     PULSE_REQUIRE((reinterpret_cast<uintptr_t>(q_w) % 16) == 0 && (reinterpret_cast<uintptr_t>(k_w) % 16) == 0 &&
                   (reinterpret_cast<uintptr_t>(cos_t) % 16) == 0 && (reinterpret_cast<uintptr_t>(sin_t) % 16) == 0,
                   "attn_decode: norm weights and rotation tables must be 16-byte aligned");
-    PULSE_REQUIRE(nq > 0 && nkv > 0 && qkv_stride >= static_cast<int64_t>(nq + (new_key ? 2 * nkv : 0)) * D,
+    PULSE_REQUIRE(nq > 0 && nkv > 0 && qkv_stride >= static_cast<int64_t>(nq + (new_key ? nkv : 0)) * D &&
+                  ((extras && extras->v_head0 >= 0) || qkv_stride >= static_cast<int64_t>(nq + (new_key ? 2 * nkv : 0)) * D),
                   "attn_decode: the projection output's rows are too short");
     PULSE_REQUIRE(n_items == tokens, "attn_decode: %d items for %d tokens (every item holds one token)", n_items, tokens);
     Preparation prep{q_w, k_w, cos_t, sin_t, eps, rotary_dim, pairing, new_key ? 1 : 0};
     return launch_attn_mfma(qkv, qkv_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items,
                             n_items, tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits,
-                            max_context, part_o, part_ml, &prep, live_context, plan, stream);
+                            max_context, part_o, part_ml, &prep, live_context, plan, extras, stream);
 }
 
 // Keys a split of the prompt-portion kernel must be a multiple of; 0 when this head size's kernel has no splits.
@@ -1698,7 +1761,8 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
                                   const void* vcache, const int* positions, const int* block_table, int bt_width,
                                   const int* items, int n_items, int tokens,
                                   int nq, int nkv, int page_size, int num_pages, float scale, int window,
-                                  int split_size, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
+                                  int split_size, int n_splits, float* part_o, float* part_ml,
+                                  const PulseAttnExtras* extras, hipStream_t stream) {
     PULSE_REQUIRE(n_splits >= 1 && n_splits < 65536, "attn_prefill: bad number of splits %d", n_splits);
     if (n_splits > 1) {
         PULSE_REQUIRE(pulse_attn_prefill_split_keys() > 0, "attn_prefill: head size %d has no split variant", D);
@@ -1736,6 +1800,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.live_context = nullptr;
     a.plan = nullptr;
     a.part_o = n_splits > 1 ? part_o : nullptr; a.part_ml = n_splits > 1 ? part_ml : nullptr;
+    if (take_gate(a, extras, nq)) return 1;
 #if PULSE_WIDE
     hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks, n_splits),
                        dim3(WIDE_NW * PULSE_WAVE), 0, stream, a, 16 / gp);
@@ -1744,7 +1809,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
         const int item_tokens = WIDE_NW * WIDE_CT * (16 / gp);
         hipLaunchKernelGGL(attn_prefill_reduce_kernel, dim3(n_items * item_tokens, (nq + PR_HEADS - 1) / PR_HEADS),
                            dim3(PR_THREADS), 0, stream, part_o, part_ml, positions, items, item_tokens, a.out, o_stride, nq,
-                           n_splits, split_size);
+                           n_splits, split_size, a.gate, a.gate_stride);
     }
 #else
     hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_items, nkv * a.head_chunks), dim3(WAVES * PULSE_WAVE), 0, stream, a,

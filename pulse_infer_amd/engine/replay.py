@@ -48,7 +48,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     _, model = load_model(args.model, mode=args.dtype, device=args.device)
     pool_tokens = (args.max_tokens + ROUND_TO - 1) // ROUND_TO * ROUND_TO
     runner = ModelRunner(model, page_size=args.page_size, num_pages=pool_tokens // args.page_size,
-                         max_requests=max(MAX_LIVE, 8))
+                         max_requests=MAX_LIVE)
     held: Dict[str, int] = {}
 
     for line in sys.stdin:

@@ -23,7 +23,9 @@ def step_cost(spec: ModelSpec, entries: List[Tuple[int, int]], wanted: int, weig
         block = BLOCKS.get(layer.block.kind)
         mixer = MIXERS.get(layer.mixer.kind).step_cost(layer.mixer.params, entries, weight_bytes, cache_bytes)
         cost = cost + mixer
-        cost = cost + FEED_FORWARDS.get(layer.ffn.kind).step_cost(layer.ffn.params, entries, weight_bytes, cache_bytes)
+        if layer.ffn is not None:
+            cost = cost + FEED_FORWARDS.get(layer.ffn.kind).step_cost(layer.ffn.params, entries, weight_bytes,
+                                                                      cache_bytes)
         for place in getattr(block, "NORM_PLACES", ()):
             norm = layer.norm(place)
             cost = cost + NORMS.get(norm.kind).step_cost(norm.params, entries, weight_bytes, cache_bytes)

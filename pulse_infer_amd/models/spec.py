@@ -36,7 +36,7 @@ class LayerSpec:
 
     prefix: str
     mixer: PartSpec
-    ffn: PartSpec
+    ffn: Optional[PartSpec]      # None: the layer has no feed-forward (for block arrangements that allow it)
     norms: Dict[str, PartSpec]
     block: PartSpec = field(default_factory=lambda: PartSpec("prenorm", {"mixer_norm": "input_layernorm",
                                                                          "ffn_norm": "post_attention_layernorm"}))

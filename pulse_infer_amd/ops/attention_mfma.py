@@ -20,6 +20,36 @@ def supported(head_dim: int, page_size: int, dtype: torch.dtype, cache_dtype: to
             and 16 <= head_dim <= MAX_HEAD_DIM and page_size % 16 == 0)
 
 
+class _Extras(ctypes.Structure):
+    # as PulseAttnExtras of the kernel source
+    _fields_ = [("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_int64), ("plain_norm", ctypes.c_int),
+                ("v_head0", ctypes.c_int), ("temp_coef", ctypes.c_float), ("temp_every", ctypes.c_int)]
+
+
+def _extras(what: str, tokens: int, nq: int, gate: Optional[torch.Tensor] = None, plain_norm: bool = False,
+            v_head0: int = -1, q_temperature: Optional[Tuple[float, int]] = None):
+    """What the entry points take besides their lists, or a null pointer when there is none of it.  ``gate``: bfloat16
+    [tokens, nq] (rows may be strided), the logits of an output gate: head h of token t leaves the kernel multiplied
+    by sigmoid(gate[t, h]).  The rest is for ``attn_decode``: a norm of q and k without weights, the head number at
+    which the raw values start in a row of the projection output, and a query temperature (coef, every):
+    q *= 1 + coef * ln(floor((position + 1) / every) + 1)."""
+    if gate is None and not plain_norm and v_head0 < 0 and q_temperature is None:
+        return None
+    ex = _Extras()
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.bfloat16 and gate.dim() == 2 and gate.shape[0] == tokens
+              and gate.shape[1] >= nq and gate.stride(1) == 1,
+              f"{what}: the gate must be bfloat16 [{tokens}, {nq}] with contiguous rows")
+        ex.gate, ex.gate_stride = gate.data_ptr(), gate.stride(0) if tokens > 1 else max(nq, gate.shape[1])
+    ex.plain_norm = 1 if plain_norm else 0
+    ex.v_head0 = int(v_head0)
+    if q_temperature is not None:
+        coef, every = q_temperature
+        _need(int(every) > 0, f"{what}: the query temperature's interval must be positive")
+        ex.temp_coef, ex.temp_every = float(coef), int(every)
+    return ctypes.byref(ex)
+
+
 def tokens_per_item(group: int) -> int:
     """How many consecutive tokens of a request share one work item (16 columns / heads per kv head)."""
     gp = 1
@@ -115,7 +145,8 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
               vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
               items: torch.Tensor, scale: float, window: int, split_size: int, n_splits: int, max_context: int,
               part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
-              live_context: Optional[torch.Tensor] = None, plan: Optional[torch.Tensor] = None) -> None:
+              live_context: Optional[torch.Tensor] = None, plan: Optional[torch.Tensor] = None,
+              gate: Optional[torch.Tensor] = None) -> None:
     """Attention of decoded tokens and short portions.  ``split_size`` x ``n_splits`` is what the launch is made for
     (contexts up to ``max_context``); ``live_context`` (one int32 on the device: the longest context among the step's
     entries as it is now) lets the kernel cut the keys that are there evenly into the same number of splits;
@@ -146,7 +177,7 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
             _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml),
-            _ptr(live_context), _ptr(plan), _stream())
+            _ptr(live_context), _ptr(plan), _extras("attn_mfma", tokens, nq, gate), _stream())
 
 
 PLAN_MIN_KEYS = 256      # no split of a plan is shorter (what a workgroup costs beside its walk, in keys walked)
@@ -263,7 +294,8 @@ def choose_prefill_splits(entries: Sequence, portion: int, nkv: int, group: int,
 def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
                  vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                  items: torch.Tensor, scale: float, window: int, split_size: int = 0, n_splits: int = 1,
-                 part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> None:
+                 part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                 gate: Optional[torch.Tensor] = None) -> None:
     """Attention for prompt portions: items of up to portion_tokens(group, d) tokens, keys shared through LDS.
     With ``n_splits > 1`` the keys are walked in splits of ``split_size`` (a multiple of 64) by workgroups of their
     own and merged by a second kernel; ``part_o`` / ``part_ml`` are float32 scratch of tokens * nq * n_splits * d
@@ -294,7 +326,8 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(items.numel() // ITEM_INTS), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
             _f32(scale), _i32(window), _i32(split_size if n_splits > 1 else 0), _i32(n_splits),
-            _ptr(part_o if n_splits > 1 else None), _ptr(part_ml if n_splits > 1 else None), _stream())
+            _ptr(part_o if n_splits > 1 else None), _ptr(part_ml if n_splits > 1 else None),
+            _extras("attn_prefill", tokens, nq, gate), _stream())
 
 
 def decode_takes(d: int, rotary_dim: int, pairing: int) -> bool:
@@ -310,10 +343,12 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
                 part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], q_w: Optional[torch.Tensor],
                 k_w: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                 rotary_dim: int, pairing: int, new_key: bool, live_context: Optional[torch.Tensor] = None,
-                plan: Optional[torch.Tensor] = None) -> None:
+                plan: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, plain_norm: bool = False,
+                v_head0: int = -1, q_temperature: Optional[Tuple[float, int]] = None) -> None:
     """Attention for decoded tokens from the raw projection output ``qkv`` [tokens, (nq + 2 nkv) d]: per-head norm
     and rotation of q and of the token's own key happen inside the kernel; with ``new_key`` key and value are also
-    written to the token's page.  Every item must hold one token; ``items`` None says that item i is token i with row
+    written to the token's page.  ``plain_norm``: the norm has no weights; ``v_head0``: the raw values start at head
+    number ``v_head0`` of a row instead of nq + nkv; ``q_temperature``, ``gate``: see ``_extras``.  Every item must hold one token; ``items`` None says that item i is token i with row
     i of the block table (a step of decoded tokens in the order of its requests), which spares every workgroup the
     trip to memory for its item.  ``live_context``, ``plan``: as for ``attn_mfma``."""
     _gpu("attn_decode", qkv, out, kcache, vcache, positions, block_table, items, part_o, part_ml, q_w, k_w, cos, sin,
@@ -323,8 +358,10 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
     _planned(plan, tokens, n_splits)
     _need(qkv.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and qkv.stride(1) == 1 and out.stride(1) == 1,
           "attn_decode: qkv and out must be bfloat16 matrices with contiguous rows")
-    _need(qkv.shape[1] >= (nq + (2 * nkv if new_key else 0)) * d and out.shape[1] >= nq * d and out.shape[0] == tokens,
-          "attn_decode: qkv/out too narrow")
+    v_end = (v_head0 if v_head0 >= 0 else nq + nkv) + nkv
+    _need(qkv.shape[1] >= (max(nq + nkv, v_end) if new_key else nq) * d and out.shape[1] >= nq * d
+          and out.shape[0] == tokens, "attn_decode: qkv/out too narrow")
+    _need(not (plain_norm and (q_w is not None or k_w is not None)), "attn_decode: a norm without weights takes none")
     pages, page_size = _check_cache("attn_decode", kcache, vcache, nkv, d)
     _need(supported(d, page_size, qkv.dtype, kcache.dtype), f"attn_decode: head size {d} / page size {page_size} / "
           f"{kcache.dtype} is not supported by the matrix-core kernel")
@@ -355,4 +392,5 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
             _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
             _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _ptr(q_w), _ptr(k_w),
             _f32(eps), _ptr(cos), _ptr(sin), _i32(rotary_dim if cos is not None else 0), _i32(pairing),
-            _i32(1 if new_key else 0), _ptr(live_context), _ptr(plan), _stream())
+            _i32(1 if new_key else 0), _ptr(live_context), _ptr(plan),
+            _extras("attn_decode", tokens, nq, gate, plain_norm, v_head0, q_temperature), _stream())

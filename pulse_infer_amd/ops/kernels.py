@@ -84,8 +84,10 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_
 
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_back: bool = True) -> None:
-    """out[r] = rmsnorm(h[s] + delta[s]) * weight, s = rows[r] or r; with write_back h[s] keeps the sum.
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_back: bool = True,
+                weight_offset: float = 0.0) -> None:
+    """out[r] = rmsnorm(h[s] + delta[s]) * (weight_offset + weight), s = rows[r] or r; with write_back h[s] keeps the
+    sum.  ``weight_offset`` is 1 for a weight stored as its distance from one (added in float32), else 0.
     ``delta`` may be float32 [parts, T, H]: the shares of a product whose inner dimension was split, added in order."""
     _gpu("add_rmsnorm", h, delta, weight, out, rows)
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "add_rmsnorm: h must be contiguous float32 [T, H]")
@@ -107,7 +109,8 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
           f"add_rmsnorm: out must be [{n_out}, {hidden}], got {tuple(out.shape)}")
     call("pulse_add_rmsnorm", _ptr(h), _ptr(delta), _i32(_tag(delta, "add_rmsnorm") if delta is not None else 0),
          _i32(parts), _i64(h.numel()), _ptr(rows), _ptr(weight), _i32(_tag(weight, "add_rmsnorm")), _ptr(out), _i32(_tag(out, "add_rmsnorm")),
-         _i32(n_out), _i32(hidden), _f32(eps), _i32(1 if (write_back and delta is not None) else 0), _stream())
+         _i32(n_out), _i32(hidden), _f32(eps), _i32(1 if (write_back and delta is not None) else 0), _f32(weight_offset),
+         _stream())
 
 
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
@@ -189,7 +192,8 @@ def gemm_skinny_fusable(m: int, n: int, k: int) -> bool:
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
                 tune: int = 0, sumsq_out: Optional[torch.Tensor] = None, row_scale: Optional[tuple] = None,
-                copy_out: Optional[torch.Tensor] = None, copy_scale: Optional[torch.Tensor] = None) -> None:
+                copy_out: Optional[torch.Tensor] = None, copy_scale: Optional[torch.Tensor] = None,
+                copy_offset: float = 0.0) -> None:
     """out = a @ w^T for at most 64 rows of bfloat16, float32 accumulation on the matrix cores.
 
     ``out`` bfloat16 or float32 is stored; with ``add`` (float32 only) the product is added to it.  With
@@ -201,8 +205,9 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
     RMSNorm moved behind the product, ``sumsq`` [M, parts] being the sums of squares, in parts, of the rows that were
     normed (the norm's weight has to be in ``a`` already).  ``sumsq_out`` [M, ceil(N / 16)] with ``add``: the kernel
     also leaves the sums of squares of the rows of the updated ``out``, 16 columns a part; ``copy_out`` [M, N] bfloat16
-    with ``add``: the updated ``out`` once more, every column multiplied by its ``copy_scale`` (bfloat16 [N], the weight
-    of the norm that reads ``out`` next; None: as it is) and rounded: what ``row_scale`` of the next product takes.
+    with ``add``: the updated ``out`` once more, every column multiplied by ``copy_offset`` + its ``copy_scale``
+    (bfloat16 [N], the weight of the norm that reads ``out`` next, and what that norm adds to its weight; None: as it
+    is) and rounded: what ``row_scale`` of the next product takes.
     """
     scale_sumsq, scale_eps = row_scale if row_scale is not None else (None, 0.0)
     _gpu("gemm_skinny", a, w, out, sumsq_out, copy_out, scale_sumsq, copy_scale)
@@ -245,7 +250,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
     call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
          _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
          _i32(tune), _ptr(scale_sumsq), _i32(scale_parts), _f32(scale_eps), _ptr(sumsq_out), _ptr(copy_out),
-         _i64(ldcopy), _ptr(copy_scale), _stream(), label=f"N={n} K={k}")
+         _i64(ldcopy), _ptr(copy_scale), _f32(copy_offset), _stream(), label=f"N={n} K={k}")
 
 
 ROWS_MAX_ROWS = 64
@@ -403,12 +408,20 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: Optional[
                k_weight: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                rotary_dim: int, pairing: int, kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor],
                positions: torch.Tensor, token_entry: torch.Tensor, block_table: Optional[torch.Tensor],
-               write_kv: bool = True) -> None:
-    """Per-head norm and rotation of q (in place) and k, and the page write of k and v."""
+               write_kv: bool = True, plain_norm: bool = False, v_head0: Optional[int] = None,
+               q_temperature: Optional[tuple] = None) -> None:
+    """Per-head norm and rotation of q (in place) and k, and the page write of k and v.  ``plain_norm``: q and k are
+    divided by their root mean square without weights; ``v_head0``: the head number at which the values start in a
+    row (default nq + nkv: behind the keys; nq: the values are the raw keys); ``q_temperature`` = (coef, every):
+    q *= 1 + coef * ln(floor((position + 1) / every) + 1) after the norm."""
     _gpu("qk_rope_kv", qkv, q_weight, k_weight, cos, sin, kcache, vcache, positions, token_entry, block_table)
     tokens = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qk_rope_kv: qkv must be [T, columns] with contiguous rows")
-    cols = (nq + 2 * nkv) * d if write_kv else nq * d
+    v_head0 = nq + nkv if v_head0 is None else int(v_head0)
+    cols = max(nq + nkv, v_head0 + nkv) * d if write_kv else nq * d
+    _need(v_head0 >= 0 and not (plain_norm and q_weight is not None), "qk_rope_kv: bad value columns or norm options")
+    temp_coef, temp_every = (float(q_temperature[0]), int(q_temperature[1])) if q_temperature is not None else (0.0, 0)
+    _need(q_temperature is None or temp_every > 0, "qk_rope_kv: the query temperature's interval must be positive")
     _need(qkv.shape[1] >= cols, f"qk_rope_kv: qkv has {qkv.shape[1]} columns, {cols} are needed")
     _int_vec("qk_rope_kv: positions", positions, tokens)
     _int_vec("qk_rope_kv: token_entry", token_entry, tokens)
@@ -436,15 +449,17 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: Optional[
          _ptr(k_weight), _i32(w_tag), _f32(eps), _ptr(cos), _ptr(sin), _i32(rotary_dim if cos is not None else 0),
          _i32(pairing), _ptr(kcache if write_kv else None), _ptr(vcache if write_kv else None), _i32(c_tag),
          _ptr(positions), _ptr(token_entry), _ptr(block_table if write_kv else None), _i32(width), _i32(tokens),
-         _i32(nq), _i32(nkv), _i32(d), _i32(page_size), _i32(pages), _i32(1 if write_kv else 0), _stream())
+         _i32(nq), _i32(nkv), _i32(d), _i32(page_size), _i32(pages), _i32(1 if write_kv else 0),
+         _i32(1 if plain_norm else 0), _i32(v_head0), _f32(temp_coef), _i32(temp_every), _stream())
 
 
 def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
                  vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
-                 scale: float, window: int = 0) -> None:
+                 scale: float, window: int = 0, gate: Optional[torch.Tensor] = None) -> None:
     """Paged causal attention, one wavefront per (token, head), float32 arithmetic.
 
     ``q`` is [T, >= nq*d] (rows may be strided, e.g. the front of a fused qkv buffer); ``out`` is [T, nq*d].
+    ``gate`` [T, nq] of q's storage type (rows may be strided): head h of token t is multiplied by sigmoid(gate[t, h]).
     """
     _gpu("attn_generic", q, out, kcache, vcache, positions, token_entry, block_table)
     tokens = q.shape[0]
@@ -456,10 +471,15 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
     _int_vec("attn_generic: token_entry", token_entry, tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "attn_generic: block_table must be contiguous int32 [entries, width]")
+    if gate is not None:
+        _gpu("attn_generic", gate)
+        _need(gate.dtype == q.dtype and gate.dim() == 2 and gate.shape[0] == tokens and gate.shape[1] >= nq
+              and gate.stride(1) == 1, f"attn_generic: the gate must be [{tokens}, {nq}] of q's storage type")
+    gate_stride = 0 if gate is None else (gate.stride(0) if tokens > 1 else max(nq, gate.shape[1]))
     call("pulse_attn_generic", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _i32(_tag(q, "attn_generic")),
          _ptr(kcache), _ptr(vcache), _i32(_tag(kcache, "attn_generic")), _ptr(positions), _ptr(token_entry),
          _ptr(block_table), _i32(block_table.shape[1]), _i32(tokens), _i32(nq), _i32(nkv), _i32(d), _i32(page_size),
-         _i32(pages), _f32(scale), _i32(window), _stream())
+         _i32(pages), _f32(scale), _i32(window), _ptr(gate), _i64(gate_stride), _stream())
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,

@@ -11,6 +11,18 @@ A window w gives lo = max(0, position - w + 1); without one lo = 0.
 The three projections are one product with the row-stacked weight (a layout
 choice); norm, rotation and the cache write are one kernel; the attention
 kernel is chosen by size and storage type.
+
+Variations, all parameters of the part:
+
+* ``values = "keys"``: there is no value projection; a token's values are its keys as projected, before the norm
+  (the cache then holds the normed keys and the raw ones);
+* ``qk_norm_weights = False``: the per-head norm of q and k has no weights (x / sqrt(mean(x^2) + eps) alone);
+* ``query_temperature = {"coef": c, "every": n}``: after the norm q is multiplied by
+  1 + c * ln(floor((position + 1) / n) + 1), in float32;
+* ``output_gate = True``: head h's output is multiplied by sigmoid(g_h), g = x Wg^T with Wg [heads, hidden] (one
+  number a token and head), before the output projection; Wg's rows ride behind the other projections in the
+  stacked weight, and the attention kernels apply the gate as they store their result;
+* ``names``: the tensors' names below the part's prefix.
 """
 from __future__ import annotations
 
@@ -21,7 +33,7 @@ import torch
 from ..cache.manager import PagedKVSpec
 from ..ops import attention_mfma, kernels
 from ..weights.store import TensorSpec
-from .base import MIXERS, BuildContext, LazyNorm, PagedCacheView, Part, StepContext, StepCost
+from .base import MIXERS, BuildContext, LazyNorm, PagedCacheView, Part, StepContext, StepCost, joined
 from .linear import Linear
 
 
@@ -30,16 +42,30 @@ class PagedAttention(Part):
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         hidden, nq, nkv, d = (params[k] for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
+        names = cls.tensor_names(params)
         specs = {
-            "q_proj.weight": TensorSpec((nq * d, hidden), fan_in=hidden),
-            "k_proj.weight": TensorSpec((nkv * d, hidden), fan_in=hidden),
-            "v_proj.weight": TensorSpec((nkv * d, hidden), fan_in=hidden),
-            "o_proj.weight": TensorSpec((hidden, nq * d), fan_in=nq * d),
+            names["q"]: TensorSpec((nq * d, hidden), fan_in=hidden),
+            names["k"]: TensorSpec((nkv * d, hidden), fan_in=hidden),
+            names["o"]: TensorSpec((hidden, nq * d), fan_in=nq * d),
         }
-        if params.get("qk_norm", False):
-            specs["q_norm.weight"] = TensorSpec((d,), kind="norm")
-            specs["k_norm.weight"] = TensorSpec((d,), kind="norm")
+        if params.get("values", "projection") == "projection":
+            specs[names["v"]] = TensorSpec((nkv * d, hidden), fan_in=hidden)
+        if params.get("output_gate", False):
+            specs[names["gate"]] = TensorSpec((nq, hidden), fan_in=hidden)
+        if params.get("qk_norm", False) and params.get("qk_norm_weights", True):
+            specs[names["q_norm"]] = TensorSpec((d,), kind="norm")
+            specs[names["k_norm"]] = TensorSpec((d,), kind="norm")
         return specs
+
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "gate": "g_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+    GATE_PAD = 16   # the gate's rows of the stacked weight are filled up with zero rows to a multiple of this, so that
+                    # the projection output's rows keep the alignment the kernels' 16-byte accesses need
+
+    @classmethod
+    def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
+        """The tensors' names below the part's prefix; ``params["names"]`` replaces any of the usual ones."""
+        return {**cls.NAMES, **params.get("names", {})}
 
     @classmethod
     def step_cost(cls, params: Dict[str, Any], entries, weight_bytes: int, cache_bytes: int) -> StepCost:
@@ -68,18 +94,43 @@ class PagedAttention(Part):
         if self.window is not None and int(self.window) <= 0:
             raise ValueError(f"an attention window must be positive, got {self.window}")
         self.qk_norm = bool(params.get("qk_norm", False))
+        self.plain_norm = self.qk_norm and not params.get("qk_norm_weights", True)
         self.eps = float(params.get("qk_norm_eps", 0.0))
+        values = params.get("values", "projection")
+        if values not in ("projection", "keys"):
+            raise ValueError(f"attention values must be 'projection' or 'keys', got '{values}'")
+        self.values_are_keys = values == "keys"
+        temperature = params.get("query_temperature")
+        self.q_temperature = None
+        if temperature is not None:
+            self.q_temperature = (float(temperature["coef"]), int(temperature["every"]))
+            if self.q_temperature[1] <= 0:
+                raise ValueError(f"query_temperature.every must be positive, got {self.q_temperature[1]}")
+        self.output_gate = bool(params.get("output_gate", False))
         self.position = params.get("position")
         self.encodings = build.positions
         if self.position is not None and self.position not in self.encodings:
             raise KeyError(f"attention refers to position encoding '{self.position}', the model defines "
                            f"{sorted(self.encodings)}")
         load = build.loader
-        self.qkv = Linear(load.get_concat([f"{prefix}.q_proj.weight", f"{prefix}.k_proj.weight",
-                                           f"{prefix}.v_proj.weight"]), build.mode)
-        self.o = Linear(load.get(f"{prefix}.o_proj.weight"), build.mode)
-        self.q_w = load.get(f"{prefix}.q_norm.weight") if self.qk_norm else None
-        self.k_w = load.get(f"{prefix}.k_norm.weight") if self.qk_norm else None
+        names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
+        stacked = [names["q"], names["k"]] + ([] if self.values_are_keys else [names["v"]])
+        # columns of the projection output: q heads, k heads, v heads (unless the values are the keys), gate
+        self.v_head0 = self.nq if self.values_are_keys else self.nq + self.nkv
+        self.kv_cols = (self.nq + self.nkv * (1 if self.values_are_keys else 2)) * self.d
+        self.gate_rows = 0
+        if self.output_gate:
+            weight = load.get_concat(stacked + [names["gate"]])
+            self.gate_rows = (self.nq + self.GATE_PAD - 1) // self.GATE_PAD * self.GATE_PAD
+            if self.gate_rows > self.nq:
+                weight = torch.cat([weight, weight.new_zeros(self.gate_rows - self.nq, self.hidden)], dim=0).contiguous()
+            self.qkv = Linear(weight, build.mode)
+        else:
+            self.qkv = Linear(load.get_concat(stacked), build.mode)
+        self.o = Linear(load.get(names["o"]), build.mode)
+        weighted = self.qk_norm and not self.plain_norm
+        self.q_w = load.get(names["q_norm"]) if weighted else None
+        self.k_w = load.get(names["k_norm"]) if weighted else None
         self.act_dtype = build.act_dtype
         self.options = build.options
 
@@ -91,33 +142,42 @@ class PagedAttention(Part):
     records_cleanly = True      # positions, tables and work lists are read on the device
 
     def forward(self, x, ctx: StepContext, cache: PagedCacheView, residual: Optional[torch.Tensor] = None,
-                next_scale: Optional[torch.Tensor] = None):
+                next_scale: Optional[torch.Tensor] = None, next_offset: float = 0.0, leave_stats: bool = True):
         tokens = x.shape[0]
         ws = ctx.workspace
         write = cache.writable
         q_cols = self.nq * self.d
-        cols = (self.nq + 2 * self.nkv) * self.d if write else q_cols
+        # a run that reads another run's cache needs its queries only (and all rows if a gate rides behind the keys)
+        rows = None if (write or self.output_gate) else q_cols
+        cols = self.qkv.out_features if rows is None else rows
         qkv = ws.buffer("attention.qkv", tokens, cols, self.act_dtype)
-        if isinstance(x, LazyNorm) and not self.qkv.takes_lazy(x, rows=None if write else q_cols):
+        if isinstance(x, LazyNorm) and not self.qkv.takes_lazy(x, rows=rows):
             x = x.materialize(ws.buffer("attention.normed", tokens, self.hidden, self.act_dtype))
-        self.qkv.forward(x, qkv, rows=None if write else q_cols)
+        self.qkv.forward(x, qkv, rows=rows)
+        gate = qkv[:, self.kv_cols:self.kv_cols + self.nq] if self.output_gate else None
         tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
         table = ctx.block_tables[cache.group]
         attn = ws.buffer("attention.out", tokens, q_cols, self.act_dtype)
         if self.decodes_from_raw(ctx, cache, qkv, tables):
             # decoded tokens only: the attention kernel prepares q and each token's own key itself
-            self.attend(qkv, attn, ctx, cache, table, raw=(tables, write))
+            self.attend(qkv, attn, ctx, cache, table, raw=(tables, write), gate=gate)
         else:
             kernels.qk_rope_kv(
                 qkv, self.nq, self.nkv, self.d, self.q_w, self.k_w, self.eps,
                 tables.cos if tables is not None else None, tables.sin if tables is not None else None,
                 tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
-                cache.keys, cache.values, ctx.positions, ctx.token_entry, table, write_kv=write)
-            self.attend(qkv, attn, ctx, cache, table)
+                cache.keys, cache.values, ctx.positions, ctx.token_entry, table, write_kv=write,
+                plain_norm=self.plain_norm, v_head0=self.v_head0, q_temperature=self.q_temperature)
+            self.attend(qkv, attn, ctx, cache, table, gate=gate)
         out = ws.buffer("attention.proj", tokens, self.hidden, self.act_dtype)
         if residual is not None:
-            return self.o.add_into(attn, residual, out, ws, next_scale)
+            return self.o.add_into(attn, residual, out, ws, next_scale, next_offset, leave_stats)
         return self.o.forward(attn, out)
+
+    def takes_lazy_input(self, x: LazyNorm, cache: PagedCacheView) -> bool:
+        """Whether ``forward`` would run its first product on rows that are not normalised yet, or compute the norm."""
+        rows = None if (cache.writable or self.output_gate) else self.nq * self.d
+        return self.qkv.takes_lazy(x, rows=rows)
 
     def uses_matrix_cores(self, q: torch.Tensor, cache: PagedCacheView) -> bool:
         return (self.options.get("attention", "auto") != "generic"
@@ -140,13 +200,14 @@ class PagedAttention(Part):
                 and attention_mfma.decode_takes(self.d, tables.rotary_dim, tables.pairing))
 
     def attend(self, q: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: PagedCacheView,
-               table: torch.Tensor, raw: Optional[tuple] = None) -> None:
+               table: torch.Tensor, raw: Optional[tuple] = None, gate: Optional[torch.Tensor] = None) -> None:
         """out = attention of the step's tokens over the cache.  ``raw = (rotation tables, write)``: q is the raw
-        projection output of decoded tokens, which the kernel prepares itself (see ``decodes_from_raw``)."""
+        projection output of decoded tokens, which the kernel prepares itself (see ``decodes_from_raw``).  ``gate``
+        [T, heads]: the logits of the output gate, applied by whichever kernel stores the result."""
         window = int(self.window) if self.window is not None else 0
         if not self.uses_matrix_cores(q, cache):
             kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                                 ctx.token_entry, table, self.scale, window)
+                                 ctx.token_entry, table, self.scale, window, gate=gate)
             return
         group = self.nq // self.nkv
         per = attention_mfma.tokens_per_item(group)
@@ -172,7 +233,8 @@ class PagedAttention(Part):
                 part_o = ctx.workspace.buffer("attention.portion_part_o", rows, self.d, torch.float32)
                 part_ml = ctx.workspace.buffer("attention.portion_part_ml", rows, 2, torch.float32)
             attention_mfma.attn_prefill(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                                        table, long_items, self.scale, window, split_size, n_splits, part_o, part_ml)
+                                        table, long_items, self.scale, window, split_size, n_splits, part_o, part_ml,
+                                        gate=gate)
         if short_items is not None:
             # a recorded step passes its context bucket as max_context: its splits must cover that
             max_context = ctx.max_context if long_items is None else short_context
@@ -208,9 +270,10 @@ class PagedAttention(Part):
                     self.scale, window, split_size, n_splits, max_context, part_o, part_ml, self.q_w, self.k_w,
                     self.eps, tables.cos if tables is not None else None, tables.sin if tables is not None else None,
                     tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
-                    new_key=write, live_context=ctx.live_context if plan is None else None, plan=plan)
+                    new_key=write, live_context=ctx.live_context if plan is None else None, plan=plan, gate=gate,
+                    plain_norm=self.plain_norm, v_head0=self.v_head0, q_temperature=self.q_temperature)
                 return
             attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                      table, short_items, self.scale, window, split_size, n_splits,
                                      max_context, part_o, part_ml,
-                                     live_context=ctx.live_context if plan is None else None, plan=plan)
+                                     live_context=ctx.live_context if plan is None else None, plan=plan, gate=gate)

@@ -194,6 +194,7 @@ class RowStats:
     sumsq: torch.Tensor
     rounded: Optional[torch.Tensor] = None
     scaled_by: Optional[torch.Tensor] = None
+    offset: float = 0.0          # what was added to every factor of ``scaled_by`` (a norm's ``weight_offset``)
 
 
 @dataclass
@@ -252,6 +253,14 @@ class ResidualStream:
         if self.pending is not None or self.stats is None or not hasattr(norm, "lazy"):
             return None
         return norm.lazy(self.h, self.stats)
+
+    def settle(self) -> None:
+        """Add the update that is still pending to ``h`` now (a caller whose next part may reuse the buffer the update
+        lies in)."""
+        if self.pending is not None:
+            from ..ops import kernels
+            kernels.residual_add(self.h, self.pending)
+            self.pending = None
 
     def push(self, delta: Any) -> None:
         """Hand over an update ([T, H], or [parts, T, H] float32 to be added in order); None or RowStats mean the part
@@ -323,4 +332,7 @@ def says(part: Any, name: str) -> bool:
 
 
 def joined(prefix: str, name: str) -> str:
+    """``prefix.name``; an empty prefix or an empty name leaves the other alone."""
+    if not name:
+        return prefix
     return f"{prefix}.{name}" if prefix else name

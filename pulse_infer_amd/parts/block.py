@@ -3,6 +3,10 @@
 ``prenorm``: h <- h + mixer(norm_a(h)); h <- h + ffn(norm_b(h))
 (reference: src/model/qwen3/model.cpp:779-923).  The additions are deferred into
 the next norm's kernel through ``ResidualStream``.
+
+``parallel``: n = norm(h); h <- h + (mixer(n) + ffn(n)): one norm, whose output both
+sublayers read; a layer may have no feed-forward (``LayerSpec.ffn`` None), then
+h <- h + mixer(norm(h)).
 """
 from __future__ import annotations
 
@@ -70,16 +74,100 @@ class PreNormBlock(Part):
     def _scale_of(norm: Any) -> Any:
         return norm.column_scale() if norm is not None and hasattr(norm, "column_scale") else None
 
+    @classmethod
+    def _told(cls, norm: Any) -> Dict[str, Any]:
+        """What a part that adds into the residual itself is told about the norm that reads the residual next: its
+        column factors, and what it adds to them if that is not zero."""
+        told = {"next_scale": cls._scale_of(norm)}
+        offset = float(getattr(norm, "weight_offset", 0.0) or 0.0) if norm is not None else 0.0
+        if offset and told["next_scale"] is not None:
+            told["next_offset"] = offset
+        return told
+
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
         x = self._input(stream, self.mixer_norm, self.mixer, ctx)
         # a part that says so may add its result into the residual itself and return None (or the new rows' statistics,
         # for which it is told the column factors of the norm that reads the residual next)
         if getattr(self.mixer, "accepts_residual", False):
-            stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h, next_scale=self._scale_of(self.ffn_norm)))
+            stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h, **self._told(self.ffn_norm)))
         else:
             stream.push(self.mixer.forward(x, ctx, cache))
         x = self._input(stream, self.ffn_norm, self.ffn, ctx)
         if getattr(self.ffn, "accepts_residual", False):
-            stream.push(self.ffn.forward(x, ctx, residual=stream.h, next_scale=self._scale_of(stream.after_block)))
+            stream.push(self.ffn.forward(x, ctx, residual=stream.h, **self._told(stream.after_block)))
+        else:
+            stream.push(self.ffn.forward(x, ctx))
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(PreNormBlock):
+    """One norm in front of mixer and feed-forward, which both read its output; their results are added to the
+    residual together.  The feed-forward may be absent.  Block parameters: ``norm``: the norm's tensor prefix below
+    the layer's.  A mixer that says ``accepts_residual`` is also handed ``leave_stats`` here, and parts that say
+    ``accepts_lazy_input`` answer ``takes_lazy_input(x, cache)``."""
+
+    NORM_PLACES = ("norm",)
+
+    @classmethod
+    def layer_weight_specs(cls, layer: LayerSpec) -> Dict[str, TensorSpec]:
+        p = layer.block.params
+        out: Dict[str, TensorSpec] = {}
+        norm = layer.norm("norm")
+        for name, spec in NORMS.get(norm.kind).weight_specs(norm.params).items():
+            out[joined(joined(layer.prefix, p["norm"]), name)] = spec
+        parts = [(layer.mixer, MIXERS)] + ([(layer.ffn, FEED_FORWARDS)] if layer.ffn is not None else [])
+        for part, registry in parts:
+            sub = joined(layer.prefix, part.params.get("prefix", ""))
+            for name, spec in registry.get(part.kind).weight_specs(part.params).items():
+                out[joined(sub, name)] = spec
+        return out
+
+    def __init__(self, layer: LayerSpec, build: BuildContext):
+        p = layer.block.params
+        norm = layer.norm("norm")
+        self.norm = NORMS.get(norm.kind)(norm.params, joined(layer.prefix, p["norm"]), build)
+        self.mixer = MIXERS.get(layer.mixer.kind)(layer.mixer.params,
+                                                  joined(layer.prefix, layer.mixer.params.get("prefix", "")), build)
+        self.ffn = None
+        if layer.ffn is not None:
+            self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
+                                                         joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
+        self.act_dtype = build.act_dtype
+
+    def records_cleanly(self) -> bool:
+        return all(says(part, "records_cleanly") for part in (self.mixer, self.ffn, self.norm) if part is not None)
+
+    def entry_norm(self) -> Any:
+        return self.norm
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+        parts = [part for part in (self.mixer, self.ffn) if part is not None]
+        # The norm's output is read twice.  It is left to the parts' first products (rows scaled behind the product)
+        # only if every part takes it that way; a part that then cannot after all computes the norm for itself.
+        x = None
+        if all(getattr(part, "accepts_lazy_input", False) and hasattr(part, "takes_lazy_input") for part in parts):
+            x = stream.lazy(self.norm)
+            # (a part that computed the norm for itself after the other has changed the residual would norm the wrong
+            # rows: so every part is asked beforehand)
+            if x is not None and not all(part.takes_lazy_input(x, cache) for part in parts):
+                x = None
+        if x is None:
+            x = stream.normed(self.norm, ctx.workspace.buffer("block.normed", ctx.num_tokens, stream.h.shape[1],
+                                                              self.act_dtype))
+        # The mixer's update first: the part that adds last is told who reads the residual next, and what it leaves
+        # about the new rows then covers both updates.
+        last = self.ffn is None
+        if getattr(self.mixer, "accepts_residual", False):
+            # (told not to leave the new rows' statistics when it is not the last to add: their buffers are the
+            # ones the feed-forward's input still lies in)
+            told = self._told(stream.after_block) if last else {"leave_stats": False}
+            stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h, **told))
+        else:
+            stream.push(self.mixer.forward(x, ctx, cache))
+        if self.ffn is None:
+            return
+        stream.settle()   # (an update handed back in a workspace buffer must not wait while the next product runs)
+        if getattr(self.ffn, "accepts_residual", False):
+            stream.push(self.ffn.forward(x, ctx, residual=stream.h, **self._told(stream.after_block)))
         else:
             stream.push(self.ffn.forward(x, ctx))

@@ -116,15 +116,19 @@ class Linear:
         return out
 
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor,
-                 workspace: Optional[Workspace] = None, next_scale: Optional[torch.Tensor] = None):
+                 workspace: Optional[Workspace] = None, next_scale: Optional[torch.Tensor] = None,
+                 next_offset: float = 0.0, leave_stats: bool = True):
         """residual += x W^T, in one of five ways.  Few rows: the kernel adds into the residual itself and None is
         returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows (their
         sums of squares and a rounded copy, multiplied column by column by ``next_scale``, the weight of the norm that
-        reads the residual next: with these the next product can do without a norm kernel before it).  17 to
+        reads the residual next, ``next_offset`` added to each in float32: with these the next product can do without a
+        norm kernel before it).  17 to
         192 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
         results [parts, rows, out] are returned as the update, which the next norm adds up in order; more rows of a
         product with a wide inner dimension and a narrow output: the same through the library's batched product.
-        Otherwise the product is written to ``scratch`` and returned for the caller to add."""
+        Otherwise the product is written to ``scratch`` and returned for the caller to add.  ``leave_stats=False``:
+        no ``RowStats`` are made (their buffers are the workspace's, one set a width: a caller that still reads the
+        set of the rows as they were before this update says so)."""
         splits, waves = self.shares_and_waves_for(x) if workspace is not None else (0, 0)
         if splits:
             rows = x.shape[0]
@@ -156,7 +160,7 @@ class Linear:
             return parts
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
-            if (workspace is not None
+            if (workspace is not None and leave_stats
                     and kernels.gemm_skinny_fusable(x.shape[0], self.out_features, self.in_features)):
                 sums = workspace.buffer(f"linear.sumsq.{self.out_features}", x.shape[0], (self.out_features + 15) // 16,
                                         torch.float32)
@@ -165,8 +169,9 @@ class Linear:
                 scaled = next_scale is not None and next_scale.dtype == torch.bfloat16 \
                     and next_scale.numel() == self.out_features and next_scale.is_contiguous()
                 kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums, copy_out=rounded,
-                                    copy_scale=next_scale if scaled else None)
-                return RowStats(sums, rounded, next_scale if scaled else None)
+                                    copy_scale=next_scale if scaled else None,
+                                    copy_offset=next_offset if scaled else 0.0)
+                return RowStats(sums, rounded, next_scale if scaled else None, next_offset if scaled else 0.0)
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
         return self.forward(x, scratch)

@@ -10,7 +10,7 @@ import torch
 
 from ..ops import kernels
 from ..weights.store import TensorSpec
-from .base import FEED_FORWARDS, BuildContext, LazyNorm, Part, StepContext
+from .base import FEED_FORWARDS, BuildContext, LazyNorm, Part, StepContext, joined
 from .linear import Linear
 
 
@@ -22,11 +22,19 @@ class GatedMLP(Part):
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         hidden, inter = params["hidden_size"], params["intermediate_size"]
+        names = cls.tensor_names(params)
         return {
-            "gate_proj.weight": TensorSpec((inter, hidden), fan_in=hidden),
-            "up_proj.weight": TensorSpec((inter, hidden), fan_in=hidden),
-            "down_proj.weight": TensorSpec((hidden, inter), fan_in=inter),
+            names["gate"]: TensorSpec((inter, hidden), fan_in=hidden),
+            names["up"]: TensorSpec((inter, hidden), fan_in=hidden),
+            names["down"]: TensorSpec((hidden, inter), fan_in=inter),
         }
+
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+    @classmethod
+    def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
+        """The tensors' names below the part's prefix; ``params["names"]`` replaces any of the usual ones."""
+        return {**cls.NAMES, **params.get("names", {})}
 
     def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
         self.hidden = int(params["hidden_size"])
@@ -35,7 +43,8 @@ class GatedMLP(Part):
         if activation != "silu":
             raise ValueError(f"gated_mlp has no kernel for activation '{activation}' (only 'silu')")
         load = build.loader
-        gate, up = load.get(f"{prefix}.gate_proj.weight"), load.get(f"{prefix}.up_proj.weight")
+        names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
+        gate, up = load.get(names["gate"]), load.get(names["up"])
         # gate and up rows alternate in slabs of 16 where the sizes allow it, so that one workgroup of the
         # few-rows product holds a gate slab and its up slab and can apply SwiGLU itself (a layout choice)
         self.slab = SLAB if (build.mode == "bfloat16" and gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
@@ -44,17 +53,21 @@ class GatedMLP(Part):
             stacked = torch.stack([gate.view(-1, SLAB, self.hidden), up.view(-1, SLAB, self.hidden)], dim=1)
             self.gate_up = Linear(stacked.reshape(2 * self.inter, self.hidden).contiguous(), build.mode)
         else:
-            self.gate_up = Linear(load.get_concat([f"{prefix}.gate_proj.weight", f"{prefix}.up_proj.weight"]), build.mode)
+            self.gate_up = Linear(load.get_concat([names["gate"], names["up"]]), build.mode)
         del gate, up
-        self.down = Linear(load.get(f"{prefix}.down_proj.weight"), build.mode)
+        self.down = Linear(load.get(names["down"]), build.mode)
         self.act_dtype = build.act_dtype
 
     accepts_residual = True
     accepts_lazy_input = True   # the first product may take rows that are not normalised yet and scale its result
     records_cleanly = True
 
+    def takes_lazy_input(self, x: LazyNorm, cache: Any = None) -> bool:
+        """Whether ``forward`` would run its first product on rows that are not normalised yet, or compute the norm."""
+        return bool(self.slab and self.gate_up.takes_lazy(x))
+
     def forward(self, x, ctx: StepContext, residual: Optional[torch.Tensor] = None,
-                next_scale: Optional[torch.Tensor] = None):
+                next_scale: Optional[torch.Tensor] = None, next_offset: float = 0.0, leave_stats: bool = True):
         tokens = x.shape[0]
         ws = ctx.workspace
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
@@ -75,5 +88,5 @@ class GatedMLP(Part):
             kernels.swiglu(gu, z, slab=self.slab)
         out = ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype)
         if residual is not None:
-            return self.down.add_into(z, residual, out, ws, next_scale)
+            return self.down.add_into(z, residual, out, ws, next_scale, next_offset, leave_stats)
         return self.down.forward(z, out)

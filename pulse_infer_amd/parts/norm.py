@@ -1,5 +1,9 @@
-"""RMSNorm: y = x / sqrt(mean(x^2) + eps) * w, float32 inside, one rounding
-(reference: src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157; layer: src/layer/rmsnorm.cpp:9-157)."""
+"""RMSNorm: y = x / sqrt(mean(x^2) + eps) * (c + w), float32 inside, one rounding
+(reference: src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157; layer: src/layer/rmsnorm.cpp:9-157).
+
+Parameters: ``size``, ``eps``; ``weight_offset`` = c (default 0: the tensor holds the factors themselves; 1: it holds
+their distances from one, and the sum is formed in float32 whatever the tensor's storage type); ``tensor``: the
+tensor's name below the norm's prefix (default "weight"; "": the prefix itself is the tensor's name)."""
 from __future__ import annotations
 
 from typing import Any, Dict, Optional
@@ -8,19 +12,21 @@ import torch
 
 from ..ops import kernels
 from ..weights.store import TensorSpec
-from .base import NORMS, BuildContext, LazyNorm, Part, RowStats
+from .base import NORMS, BuildContext, LazyNorm, Part, RowStats, joined
 
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((params["size"],), kind="norm")}
+        kind = "norm_offset" if float(params.get("weight_offset", 0.0)) == 1.0 else "norm"
+        return {params.get("tensor", "weight"): TensorSpec((params["size"],), kind=kind)}
 
     def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
         self.size = int(params["size"])
         self.eps = float(params["eps"])
-        self.weight = build.loader.get(f"{prefix}.weight")
+        self.weight_offset = float(params.get("weight_offset", 0.0))
+        self.weight = build.loader.get(joined(prefix, params.get("tensor", "weight")))
 
     records_cleanly = True
     takes_parts = True   # delta may be [parts, T, H] float32: the kernel adds the parts in order
@@ -28,17 +34,18 @@ class RMSNorm(Part):
     def apply(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: torch.Tensor,
               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """out = norm(h + delta) * w; h keeps the sum unless rows are gathered."""
-        kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows)
+        kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows, weight_offset=self.weight_offset)
         return out
 
     def column_scale(self) -> Optional[torch.Tensor]:
-        """The factor of every column: whoever writes the rows that this norm reads next may multiply it in as it
-        writes a rounded copy of them (``RowStats``), and leave the rest of the norm to the consumer."""
+        """The factor of every column (plus ``weight_offset``): whoever writes the rows that this norm reads next may
+        multiply it in as it writes a rounded copy of them (``RowStats``), and leave the rest of the norm to the
+        consumer."""
         return self.weight
 
     def lazy(self, h: torch.Tensor, stats: RowStats) -> Optional[LazyNorm]:
         """This norm as an input that its consumer finishes: the rows already carry this norm's weight, and dividing
         a row by a number commutes with a linear product."""
-        if stats.rounded is None or stats.scaled_by is not self.weight:
+        if stats.rounded is None or stats.scaled_by is not self.weight or stats.offset != self.weight_offset:
             return None
         return LazyNorm(stats.rounded, stats.sumsq, self.eps, h, self)

@@ -4,7 +4,7 @@ Every tensor has a generator of its own, seeded from (seed, tensor name), so a
 tensor's values do not depend on which other tensors exist or in which order
 they are made.  Linear and embedding weights are normal with standard deviation
 1/sqrt(fan_in) (``init="fan_in"``) or a fixed one (``init=0.02``); norm weights
-are 1 + U(-0.1, 0.1).  Values are rounded to the storage type once.
+are 1 + U(-0.1, 0.1), those stored as distances from one U(-0.2, 0.2).  Values are rounded to the storage type once.
 ``write_model_folder`` writes config.json and model.safetensors; ``RandomSource``
 serves the same tensors without a file (for sizes not worth writing to disk).
 (The reference has no such mode; its tests seed tensors by hand,
@@ -37,6 +37,8 @@ def make_tensor(name: str, spec: TensorSpec, seed: int, init: Init = "fan_in",
     shape = tuple(spec.shape)
     if spec.kind == "norm":
         t = 1.0 + (torch.rand(shape, generator=gen, device=device, dtype=torch.float32) * 0.2 - 0.1)
+    elif spec.kind == "norm_offset":   # a norm weight stored as its distance from one
+        t = torch.rand(shape, generator=gen, device=device, dtype=torch.float32) * 0.4 - 0.2
     elif spec.kind == "table":
         return torch.randint(0, 2 ** 15, shape, generator=gen, device=device, dtype=torch.int32)
     else:

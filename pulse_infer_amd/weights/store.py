@@ -40,6 +40,7 @@ class TensorSpec:
 
     ``kind`` drives random initialisation: ``linear`` and ``embedding`` are
     normal with a scale from ``fan_in``; ``norm`` is 1 + U(-0.1, 0.1);
+    ``norm_offset`` (a norm weight stored as its distance from one) is U(-0.2, 0.2);
     ``table`` is an integer table.
     """
 
