@@ -1,0 +1,600 @@
+"""Dirozen on the GPU against the plain implementation (tests/plain/dirozen_plain.py), in 32-bit and in bfloat16.
+
+Small configurations of their own and seeded random weights: layers that differ from each other (grouped and
+ungrouped heads, head sizes 16 to 128, with and without a feed-forward, temperature intervals from 5 positions on so
+that its steps fall inside prompts, inside portions and between decoded tokens), one configuration whose sizes
+coincide (heads x head size = width = feed-forward width, one head a key/value head) and one with the widths at
+which the serving kernels fuse the norm into the products.  Each mechanism alone at the kernels; then whole prompts,
+token-by-token decoding, portions down to two tokens, mixed batches with pages used again, a far key that stands
+out, long decoding through recorded steps, and greedy generation through the scheduler.
+"""
+import math
+import random
+
+import pytest
+import torch
+
+from conftest import token_ids
+from plain import dirozen_plain as P
+from test_gpu_model import SPLIT_TOL, TOL, close, mixed_trace, pages_were_used_again, run_alone, run_mixed
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F64 = torch.float64
+
+
+def layer(heads, kv_heads, dim, scale, coef, every, ff):
+    return {"type": "attention",
+            "mixer": {"dim": dim, "heads": heads, "kv_heads": kv_heads, "q_temp": {"coef": coef, "every": every},
+                      "scale": scale, "vdim": dim},
+            "mlp": None if ff is None else {"ff": ff, "kind": "dense"}}
+
+
+def config(vocab, width, eps, layers):
+    return {"architecture": "Dirozen", "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
+# every layer another shape: three cache groups, a layer without a feed-forward, head size 48 (no power of two)
+MIXED = config(301, 96, 1e-5, [layer(6, 2, 32, 0.2, 0.25, 7, 160), layer(4, 4, 16, 0.3, 0.5, 16, None),
+                               layer(3, 1, 48, 0.11, 0.1, 5, 224)])
+# sizes that coincide: heads x head size = width = feed-forward width, a key/value head a query head, equal layers
+EQUAL = config(515, 128, 1e-6, [layer(2, 2, 64, 0.125, 0.3, 32, 128)] * 2)
+# widths at which decoding steps fuse the norm into the products (inner sizes that are multiples of 1,024), a
+# feed-forward as wide as the heads together, a layer without one, grouped heads of 128
+WIDE = config(300, 1024, 1e-6, [layer(8, 2, 128, 0.09, 0.3, 24, 1024), layer(8, 8, 128, 0.07, 0.2, 9, None),
+                                layer(16, 4, 64, 0.12, 0.4, 40, 2048)])
+CONFIGS = {"mixed": MIXED, "equal": EQUAL, "wide": WIDE}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.config import DirozenConfig
+    from pulse_infer_amd.weights import write_model_folder
+
+    out = {}
+    for seed, (name, cfg) in enumerate(CONFIGS.items()):
+        out[name] = write_model_folder(DirozenConfig.from_dict(cfg), str(tmp_path_factory.mktemp(name)), seed=70 + seed)
+    return out
+
+
+@pytest.fixture(scope="module")
+def plain(folders):
+    models = {name: P.PlainDirozen.from_folder(folder) for name, folder in folders.items()}
+    memo = {}
+
+    def logits(name, ids):
+        key = (name, tuple(ids))
+        if key not in memo:
+            memo[key] = models[name].logits(list(ids))
+        return memo[key]
+
+    logits.models = models
+    return logits
+
+
+@pytest.fixture(scope="module")
+def runners(folders):
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+
+    made = {}
+
+    def get(name, dtype, page=16, tokens=512):
+        key = (name, dtype, page, tokens)
+        if key not in made:
+            _, model = load_model(folders[name], mode=dtype)
+            made[key] = ModelRunner(model, page_size=page, num_pages=tokens // page, max_requests=4)
+        return made[key]
+
+    return get
+
+
+# ------------------------------------------------------------------------------------------- mechanisms alone
+def rnd(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float32) * scale
+
+
+def stored(x, dtype):
+    dev = x.to(dtype).to(DEV)
+    return dev, dev.cpu().to(F64)
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [96, 1000, 2048])
+def test_norm_with_a_weight_stored_around_zero(dtype, hidden):
+    """x / sqrt(mean(x^2) + eps) * (1 + w): the one is added in float32, so a weight of 2^-9, which bfloat16 cannot
+    add to one, still shows."""
+    from pulse_infer_amd.ops import kernels
+
+    rows, eps = 5, 3e-6
+    h = rnd(rows, hidden, seed=1, scale=3.0).to(DEV)
+    delta, dref = stored(rnd(rows, hidden, seed=2), dtype)
+    weight = rnd(hidden, seed=3, scale=0.2)
+    weight[::3] = 2.0 ** -9
+    w, wref = stored(weight, dtype)
+    out = torch.empty(rows, hidden, dtype=dtype, device=DEV)
+    want_h = h.cpu().to(F64) + dref
+    kernels.add_rmsnorm(h, delta, w, eps, out, weight_offset=1.0)
+    want = P.offset_norm(want_h, wref, eps)
+    assert torch.allclose(out.cpu().to(F64), want, **tol(dtype))
+    assert torch.allclose(h.cpu().to(F64), want_h, atol=1e-6)
+    if dtype == torch.float32:
+        without = P.unit_rms(want_h, eps)     # (1 + 2^-9 must not have collapsed to 1)
+        assert float((out.cpu().to(F64) - without)[:, ::3].abs().min()) > 0
+
+
+def paged(lens, nkv, d, bs, dtype, seed):
+    """Empty pages (filled with NaN: nothing stale may reach an output) and a shuffled block table for requests with
+    contexts ``lens``."""
+    pages_per = [(n + bs - 1) // bs for n in lens]
+    total = sum(pages_per) + 2
+    perm = torch.randperm(total, generator=torch.Generator().manual_seed(seed)).tolist()
+    kc = torch.full((total, nkv, bs, d), float("nan"), dtype=dtype, device=DEV)
+    vc = torch.full((total, nkv, d, bs), float("nan"), dtype=dtype, device=DEV)
+    table = torch.full((len(lens), max(pages_per)), -1, dtype=torch.int32)
+    at = 0
+    for r, n in enumerate(pages_per):
+        table[r, :n] = torch.tensor(perm[at:at + n], dtype=torch.int32)
+        at += n
+    return kc, vc, table
+
+
+def attention_rows(q, keys, values, gate, positions, entry, scale, share):
+    """softmax(q . k * scale) v * sigmoid(gate) per token and head, float64; keys / values per request [S, G, d]."""
+    out = torch.zeros_like(q)
+    for t, (p, e) in enumerate(zip(positions, entry)):
+        for h in range(q.shape[1]):
+            g = h // share
+            w = torch.softmax((keys[e][:p + 1, g] @ q[t, h]) * scale, dim=0)
+            out[t, h] = (w.view(-1, 1) * values[e][:p + 1, g]).sum(0) * torch.sigmoid(gate[t, h])
+    return out
+
+
+ATTENTION_CASES = [
+    dict(nq=6, nkv=2, d=32, bs=16, lens=[150, 1, 64, 65], portion=70, every=7),
+    dict(nq=4, nkv=4, d=64, bs=16, lens=[300, 33, 17], portion=129, every=64),
+    dict(nq=8, nkv=2, d=128, bs=32, lens=[257, 100], portion=40, every=100),
+    dict(nq=3, nkv=1, d=48, bs=16, lens=[97, 40, 5], portion=2, every=5),
+    dict(nq=2, nkv=1, d=20, bs=4, lens=[45, 9], portion=11, every=3),        # sizes only the element-wise kernels take
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATTENTION_CASES)
+@pytest.mark.parametrize("path", ["generic", "matrix", "matrix_splits", "portion", "portion_splits"])
+def test_attention_with_keys_as_values_temperature_and_gate(case, path, dtype):
+    """One step of a portion of request 0 beside single tokens of the others, over pages that hold the earlier
+    tokens: the preparation kernel (norm without weights, temperature by position, the raw key as the value) and each
+    attention kernel with the gate in its store (directly, and behind the merge of splits)."""
+    from pulse_infer_amd.ops import attention_mfma as M
+    from pulse_infer_amd.ops import kernels
+
+    nq, nkv, d, bs, lens, portion, every = (case[x] for x in ("nq", "nkv", "d", "bs", "lens", "portion", "every"))
+    if path != "generic" and (dtype != torch.bfloat16 or not M.supported(d, bs, dtype, dtype)):
+        pytest.skip("the matrix-core kernels take bfloat16, head sizes in steps of 16 and pages of 16 and more")
+    if path == "portion_splits" and d not in M.PREFILL_SPLIT_HEAD_DIMS:
+        pytest.skip("this head size's portion kernel has no splits")
+    eps, coef, scale, share = 1e-5, 0.35, 0.21, nq // nkv
+    kc, vc, table = paged(lens, nkv, d, bs, dtype, seed=3)
+    gate_rows = 16
+    cols = (nq + nkv) * d + gate_rows
+    # earlier tokens of every request, through the same preparation kernel in steps of their own
+    raw_k, history = [], []
+    for r, n in enumerate(lens):
+        rows, ref = stored(rnd(n, cols, seed=10 + r), dtype)
+        raw_k.append(ref[:, nq * d:(nq + nkv) * d].reshape(n, nkv, d))
+        history.append(rows)
+    fed = [lens[0] - portion] + [n - 1 for n in lens[1:]]
+    for r, n in enumerate(fed):
+        if n:
+            kernels.qk_rope_kv(history[r][:n].clone(), nq, nkv, d, None, None, eps, None, None, 0, 0, kc, vc,
+                               torch.arange(n, dtype=torch.int32, device=DEV),
+                               torch.full((n,), r, dtype=torch.int32, device=DEV), table.to(DEV),
+                               plain_norm=True, v_head0=nq, q_temperature=(coef, every))
+    # the step
+    positions = list(range(fed[0], lens[0])) + [n - 1 for n in lens[1:]]
+    entry = [0] * portion + list(range(1, len(lens)))
+    step = torch.cat([history[0][fed[0]:]] + [history[r][n - 1:] for r, n in enumerate(lens) if r]).contiguous()
+    ref = step.cpu().to(F64)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    ent_t = torch.tensor(entry, dtype=torch.int32, device=DEV)
+    kernels.qk_rope_kv(step, nq, nkv, d, None, None, eps, None, None, 0, 0, kc, vc, pos_t, ent_t, table.to(DEV),
+                       plain_norm=True, v_head0=nq, q_temperature=(coef, every))
+    assert torch.equal(step[:, nq * d:], ref.to(dtype).to(DEV)[:, nq * d:])       # keys and gate columns stay raw
+    q_want = P.unit_rms(ref[:, :nq * d].reshape(-1, nq, d), eps) * \
+        P.query_temperature(positions, coef, every).view(-1, 1, 1)
+    assert torch.allclose(step[:, :nq * d].cpu().to(F64).reshape(-1, nq, d), q_want, **tol(dtype))
+    assert len({(p + 1) // every for p in positions}) > 1, "the step should cross a temperature step"
+    keys = [P.unit_rms(k, eps).to(dtype).to(F64) for k in raw_k]                  # stored rounded
+    for r, n in enumerate(lens):                                                  # the pages hold exactly that
+        for j in (0, n // 2, n - 1):
+            page, slot = int(table[r, j // bs]), j % bs
+            assert torch.allclose(kc[page, :, slot, :].cpu().to(F64), keys[r][j], **tol(dtype))
+            assert torch.equal(vc[page, :, :, slot].cpu().to(F64), raw_k[r][j])
+    gate = step[:, (nq + nkv) * d:(nq + nkv) * d + nq]
+    q_used = step[:, :nq * d].cpu().to(F64).reshape(-1, nq, d)
+    want = attention_rows(q_used, keys, raw_k, gate.cpu().to(F64), positions, entry, scale, share)
+    out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
+    if path == "generic":
+        kernels.attn_generic(step, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), scale, 0, gate=gate)
+    else:
+        class E:
+            def __init__(self, first_row, count):
+                self.first_row, self.count = first_row, count
+        numbered = list(enumerate([E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)]))
+        scratch = lambda splits: (torch.full((len(positions) * nq * splits, d), float("nan"), device=DEV),
+                                  torch.full((len(positions) * nq * splits, 2), float("nan"), device=DEV))
+        small = numbered
+        if path.startswith("portion"):
+            small = numbered[1:]
+            big = torch.tensor(M.build_items(numbered[:1], M.portion_tokens(share, d)), dtype=torch.int32, device=DEV)
+            if path == "portion_splits":
+                n_big = (lens[0] + 63) // 64
+                M.attn_prefill(step, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), big, scale, 0, 64, n_big,
+                               *scratch(n_big), gate=gate)
+            else:
+                M.attn_prefill(step, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), big, scale, 0, gate=gate)
+        items = torch.tensor(M.build_items(small, M.tokens_per_item(share)), dtype=torch.int32, device=DEV)
+        split = 32 if path == "matrix_splits" else (max(lens) + 31) // 32 * 32
+        n_splits = (max(lens) + split - 1) // split
+        M.attn_mfma(step, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, 0, split, n_splits, max(lens),
+                    *scratch(n_splits), gate=gate)
+    got = out.cpu().to(F64).reshape(-1, nq, d)
+    assert torch.allclose(got, want, **tol(dtype)), float((got - want).abs().max())
+
+
+@pytest.mark.parametrize("case", [c for c in ATTENTION_CASES if c["d"] % 16 == 0 and c["bs"] % 16 == 0])
+@pytest.mark.parametrize("split", [None, 32])
+def test_decoded_tokens_from_the_raw_projection(case, split):
+    """The kernel for decoded tokens that prepares q and the token's own key itself: norm without weights, the
+    temperature of the token's position, the raw key as its value, the gate; and it leaves the pages as the
+    preparation kernel does."""
+    from pulse_infer_amd.ops import attention_mfma as M
+    from pulse_infer_amd.ops import kernels
+
+    nq, nkv, d, bs, every = (case[x] for x in ("nq", "nkv", "d", "bs", "every"))
+    lens = case["lens"] + [every, every - 1 if every > 1 else 2, 2 * every]     # positions around the temperature's steps
+    dtype, eps, coef, scale, share, n = torch.bfloat16, 1e-5, 0.35, 0.21, nq // nkv, len(lens)
+    kc, vc, table = paged(lens, nkv, d, bs, dtype, seed=4)
+    cols = (nq + nkv) * d + 16
+    raw_k, last = [], []
+    for r, c in enumerate(lens):
+        rows, ref = stored(rnd(c, cols, seed=20 + r), dtype)
+        raw_k.append(ref[:, nq * d:(nq + nkv) * d].reshape(c, nkv, d))
+        if c > 1:
+            kernels.qk_rope_kv(rows[:c - 1].clone(), nq, nkv, d, None, None, eps, None, None, 0, 0, kc, vc,
+                               torch.arange(c - 1, dtype=torch.int32, device=DEV),
+                               torch.full((c - 1,), r, dtype=torch.int32, device=DEV), table.to(DEV),
+                               plain_norm=True, v_head0=nq, q_temperature=(coef, every))
+        last.append(rows[c - 1:])
+    step = torch.cat(last).contiguous()
+    ref = step.cpu().to(F64)
+    positions = [c - 1 for c in lens]
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    max_ctx = max(lens)
+    split_size, n_splits = M.choose_splits(n, nkv, share, max_ctx) if split is None else (split, (max_ctx + split - 1) // split)
+    part_o = torch.full((n * nq * n_splits, d), float("nan"), device=DEV)
+    part_ml = torch.full((n * nq * n_splits, 2), float("nan"), device=DEV)
+    out = torch.zeros(n, nq * d, dtype=dtype, device=DEV)
+    gate = step[:, (nq + nkv) * d:(nq + nkv) * d + nq]
+    M.attn_decode(step, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), None, scale, 0, split_size, n_splits, max_ctx,
+                  part_o, part_ml, None, None, eps, None, None, 0, 0, True, gate=gate, plain_norm=True, v_head0=nq,
+                  q_temperature=(coef, every))
+    assert torch.equal(step.cpu().to(F64), ref)                                   # the projection output stays raw
+    q = (P.unit_rms(ref[:, :nq * d].reshape(n, nq, d), eps)
+         * P.query_temperature(positions, coef, every).view(-1, 1, 1)).to(dtype).to(F64)
+    keys = [P.unit_rms(k, eps).to(dtype).to(F64) for k in raw_k]
+    want = attention_rows(q, keys, raw_k, gate.cpu().to(F64), positions, list(range(n)), scale, share)
+    got = out.cpu().to(F64).reshape(n, nq, d)
+    assert torch.allclose(got, want, atol=2e-2, rtol=2e-2), float((got - want).abs().max())
+    for r, p in enumerate(positions):                                             # the token's key and value in its page
+        page, slot = int(table[r, p // bs]), p % bs
+        assert torch.allclose(kc[page, :, slot, :].cpu().to(F64), keys[r][p], atol=2e-2, rtol=2e-2)
+        assert torch.equal(vc[page, :, :, slot].cpu().to(F64), raw_k[r][p])
+
+
+def test_rows_for_the_next_norm_carry_one_plus_the_weight():
+    """The few-rows product that adds into the residual leaves the new rows once more, multiplied by the next norm's
+    factors: for a weight stored around zero these are 1 + w, the one added in float32."""
+    from pulse_infer_amd.ops import kernels
+
+    m, n, kk = 5, 1024, 2048
+    a, aref = stored(rnd(m, kk, seed=1, scale=0.2), torch.bfloat16)
+    w, wref = stored(rnd(n, kk, seed=2, scale=kk ** -0.5), torch.bfloat16)
+    h = rnd(m, n, seed=3).to(DEV)
+    href = h.cpu().to(F64)
+    scale, sref = stored(rnd(n, seed=4, scale=0.2), torch.bfloat16)
+    sums = torch.zeros(m, n // 16, device=DEV)
+    copy = torch.zeros(m, n, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_skinny(a, w, h, add=True, sumsq_out=sums, copy_out=copy, copy_scale=scale, copy_offset=1.0)
+    new = href + aref @ wref.T
+    assert torch.allclose(h.cpu().to(F64), new, atol=1e-3, rtol=1e-3)
+    assert torch.allclose(copy.cpu().to(F64), new * (1.0 + sref), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(sums.sum(1).cpu().to(F64), (new * new).sum(1), rtol=1e-3)
+
+
+# ------------------------------------------------------------------------------------------------ whole models
+LENGTH = {"mixed": 150, "equal": 170, "wide": 90}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("mixed", 16), ("mixed", 4), ("equal", 16), ("equal", 64), ("wide", 16)])
+def test_whole_tail_and_portions(runners, plain, name, page, dtype):
+    ids = token_ids(CONFIGS[name]["vocab"], LENGTH[name], seed=3)
+    want = plain(name, ids)
+    runner = runners(name, dtype, page)
+    n = len(ids)
+    whole = run_alone(runner, ids, [n])
+    close(whole, want, dtype, f"{name} whole")
+    tail = run_alone(runner, ids, [n - 40] + [1] * 40)               # prefill against token-by-token decoding
+    close(tail, want, dtype, f"{name} tail")
+    close(tail, whole, dtype, f"{name} tail against whole", SPLIT_TOL)
+    for cuts in ([2, 3, 31, 2, 17, n - 57, 2], [1, 1, 1, 31, n - 34], [n - 2, 2]):
+        portions = run_alone(runner, ids, cuts)
+        close(portions, want, dtype, f"{name} portions {cuts}")
+        close(portions, whole, dtype, f"{name} portions against whole", SPLIT_TOL)
+    first = run_alone(runner, ids[:3], [1, 1, 1])                     # the first tokens of a sequence
+    close(first, want[:3], dtype, f"{name} first tokens")
+
+
+@pytest.mark.parametrize("name", ["mixed", "equal"])
+def test_the_residual_after_every_layer(runners, plain, name):
+    """Layer by layer in 32-bit: the model's own step with the residual read off behind every block."""
+    from pulse_infer_amd.engine.runner import StepEntry
+
+    ids = token_ids(CONFIGS[name]["vocab"], 37, seed=8)
+    runner = runners(name, "float32")
+    model, seen = runner.model, []
+    originals = [b.forward for b in model.blocks]
+
+    def watched(forward):
+        def run(stream, ctx, cache):
+            forward(stream, ctx, cache)
+            stream.settle()
+            seen.append(stream.h.clone())
+        return run
+
+    try:
+        for block, forward in zip(model.blocks, originals):
+            block.forward = watched(forward)
+        runner.add_request("layers")
+        runner.reserve("layers", len(ids))
+        runner.step([StepEntry("layers", ids, [])])
+    finally:
+        for block, forward in zip(model.blocks, originals):
+            block.forward = forward
+        runner.free_request("layers")
+    want = plain.models[name].residuals(ids)
+    assert len(seen) == len(want)
+    for i, (got, ref) in enumerate(zip(seen, want)):
+        close(got, ref, "float32", f"{name} after layer {i}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("mixed", 16), ("equal", 16), ("equal", 32), ("wide", 16)])
+def test_mixed_batches_with_page_reuse(runners, plain, name, page, dtype):
+    """Up to four live requests over a pool of 256 tokens, portions of some beside single tokens of others: every
+    request's logits are what it gets alone, whatever shares its steps and whoever held its pages before."""
+    ids, steps = mixed_trace(CONFIGS[name]["vocab"], seed=6, sizes=(2, 3, 5, 8, 13, 21, 34))
+    runner = runners(name, dtype, page, tokens=256)
+    got, pages_seen, most_live = run_mixed(runner, steps)
+    assert most_live == 4 and pages_were_used_again(pages_seen)
+    assert any(len(e["tokens"]) > 1 for s in steps for e in s["entries"]) and \
+        any(len(e["tokens"]) == 1 and len(s["entries"]) > 1 for s in steps for e in s["entries"])
+    for k, mine in got.items():
+        close(mine, plain(name, ids[k]), dtype, f"{name} mixed request {k}")
+
+
+def test_slots_and_pages_are_used_again_by_requests_of_other_lengths(runners, plain):
+    """Ten requests one after the other and two at a time through four slots and a pool that holds little more than
+    the two longest: a request's result does not depend on what lay in its pages before."""
+    from pulse_infer_amd.engine.runner import StepEntry
+
+    name = "mixed"
+    runner = runners(name, "float32", 16, tokens=160)
+    lengths = [70, 3, 64, 17, 1, 80, 33, 16, 65, 48]
+    for i in range(0, len(lengths), 2):
+        pair = {f"q{i + j}": token_ids(CONFIGS[name]["vocab"], n, seed=40 + i + j) for j, n in enumerate(lengths[i:i + 2])}
+        for rid, ids in pair.items():
+            runner.add_request(rid)
+            runner.reserve(rid, len(ids))
+        logits = runner.step([StepEntry(rid, ids, [len(ids) - 1]) for rid, ids in pair.items()])
+        for row, (rid, ids) in enumerate(pair.items()):
+            close(logits[row:row + 1], plain(name, ids)[-1:], "float32", f"request {rid} of {len(ids)} tokens")
+            runner.free_request(rid)
+        runner.cache.check()
+
+
+# ------------------------------------------------------------------------------ a key that stands out, far away
+NEEDLE, LAST = 650, 600
+
+
+def needle_folder(tmp_path):
+    """A one-layer model in which the query of token LAST points at the key of token NEEDLE and at no other: the key
+    projection is the query projection with its columns moved on by one, NEEDLE's embedding is LAST's moved back by
+    one (the norm's weight is zero, so the norm commutes with that), and the scale is large.  Among hundreds of keys
+    the one occurrence of NEEDLE then takes nearly all of LAST's weight, and its value decides the output."""
+    from pulse_infer_amd.config import DirozenConfig
+    from pulse_infer_amd.models.causal_lm import expected_tensors
+    from pulse_infer_amd.weights import write_safetensors
+    from pulse_infer_amd.weights.random_init import RandomSource
+
+    import json
+    import os
+
+    cfg = config(700, 64, 1e-6, [layer(2, 2, 32, 0.6, 0.2, 50, 96)])
+    typed = DirozenConfig.from_dict(cfg)
+    source = RandomSource(expected_tensors(typed.model_spec()), seed=5)
+    tensors = {name: source.get(name) for name in source.names()}
+    tensors["l0.norm1"] = torch.zeros_like(tensors["l0.norm1"])
+    tensors["l0.mix.k"] = torch.roll(tensors["l0.mix.q"], -1, dims=1).contiguous()
+    tensors["embed"][NEEDLE] = torch.roll(tensors["embed"][LAST], -1)
+    folder = str(tmp_path / "needle")
+    os.makedirs(folder, exist_ok=True)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as fh:
+        json.dump(typed.to_dict(), fh)
+    return folder
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_far_key_decides_the_output(tmp_path, dtype):
+    """The needle at position 2, at a page's last slot, at a page's first slot and one before the query, looked for
+    from the end of a prompt of 600 tokens, from a portion's last token, and from a decoded token: the logits are the
+    plain implementation's, and they are far from what they would be had the needle been missed."""
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+
+    page, n = 16, 600
+    folder = needle_folder(tmp_path)
+    oracle = P.PlainDirozen.from_folder(folder)
+    _, model = load_model(folder, mode=dtype)
+    runner = ModelRunner(model, page_size=page, num_pages=(n + page - 1) // page + 1, max_requests=2)
+    base = list(range(1, n + 1))                       # all tokens different, the last one is LAST
+    assert base[-1] == LAST
+    for where in (2, 5 * page - 1, 5 * page, n - 2):
+        ids = list(base)
+        ids[where] = NEEDLE
+        want = oracle.logits(ids)
+        missed = oracle.logits(base)
+        scale = float(want[-1].abs().max())
+        assert float((want[-1] - missed[-1]).abs().max()) > 10 * TOL[dtype] * scale, "the needle does not show"
+        for cuts in ([n], [n - 1, 1], [n - 40, 40], [where + 1, n - where - 2, 1] if where < n - 2 else [n - 3, 2, 1]):
+            got = run_alone(runner, ids, cuts)
+            close(got[-1:], want[-1:], dtype, f"needle at {where}, cuts {cuts}")
+            close(got, want, dtype, f"needle at {where}, cuts {cuts}, all positions")
+
+
+# ------------------------------------------------------------------------------------------------ long decoding
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+def test_long_decoding_of_three_requests(runners, plain, name, dtype):
+    """Three requests of unequal prompts decode 150 tokens together, one a step each, over page borders and over
+    many steps of the temperature; in bfloat16 the steps are recorded and replayed."""
+    from pulse_infer_amd.engine.runner import StepEntry
+
+    vocab, new = CONFIGS[name]["vocab"], 150
+    runner = runners(name, dtype, 16, tokens=704)
+    ids = {f"d{i}": token_ids(vocab, n + new, seed=60 + i) for i, n in enumerate((1, 30, 47))}
+    prompt = {"d0": 1, "d1": 30, "d2": 47}
+    replays = runner.graph_replays
+    got = {k: [] for k in ids}
+    for k in ids:
+        runner.add_request(k)
+        runner.reserve(k, prompt[k])
+    first = runner.step([StepEntry(k, ids[k][:prompt[k]], [prompt[k] - 1]) for k in ids])
+    for row, k in enumerate(ids):
+        got[k].append(first[row:row + 1])
+    for step in range(new):
+        for k in ids:
+            runner.reserve(k, prompt[k] + step + 1)
+        logits = runner.step([StepEntry(k, [ids[k][prompt[k] + step]], [0]) for k in ids])
+        for row, k in enumerate(ids):
+            got[k].append(logits[row:row + 1])
+    for k in ids:
+        runner.free_request(k)
+        close(torch.cat(got[k]), plain(name, ids[k])[prompt[k] - 1:], dtype, f"{name} decoding request {k}")
+    if dtype == "bfloat16":
+        assert runner.graph_replays > replays, "no decoding step was replayed from a recording"
+
+
+# --------------------------------------------------------------------------- generation through the scheduler
+@pytest.mark.parametrize("name", ["mixed", "equal"])
+def test_greedy_generation_through_the_engine(folders, plain, name):
+    """In 32-bit the greedy choice does not depend on the batch: requests generated together, in small portions and
+    with a pool so tight that some are preempted and recomputed, give what each gives alone and what the plain
+    implementation chooses."""
+    from pulse_infer_amd import LLM
+
+    vocab, new, page = CONFIGS[name]["vocab"], 12, 16
+    prompts = [token_ids(vocab, n, seed=80 + i) for i, n in enumerate((1, 5, 18, 40, 77))]
+    make = lambda **kw: LLM.from_pretrained(folders[name], dtype="float32", page_size=page, **kw)
+    alone = [make(max_batch_size=1, chunk_size=256, num_pages=32).generate([p], max_new_tokens=new, ignore_eos=True)[0]
+             for p in prompts]
+    assert alone == [plain.models[name].greedy(p, new) for p in prompts]
+    roomy = make(max_batch_size=4, chunk_size=16, num_pages=64, max_num_batched_tokens=24)
+    assert roomy.generate(prompts, max_new_tokens=new, ignore_eos=True) == alone
+    need = max((len(p) + new + page - 1) // page for p in prompts)
+    tight = make(max_batch_size=4, chunk_size=16, num_pages=need + 2)
+    assert tight.generate(prompts, max_new_tokens=new, ignore_eos=True) == alone
+    tight.engine.runner.cache.check()
+
+
+def test_bfloat16_generation_stays_within_rounding_of_the_plain_choice(folders, plain):
+    """Along the engine's own path every chosen token is the plain implementation's best one or within bfloat16's
+    error of it."""
+    from pulse_infer_amd import LLM
+
+    name, new = "wide", 10
+    prompts = [token_ids(CONFIGS[name]["vocab"], n, seed=90 + i) for i, n in enumerate((3, 21))]
+    llm = LLM.from_pretrained(folders[name], dtype="bfloat16", max_batch_size=2, chunk_size=8, page_size=16, num_pages=32)
+    for prompt, out in zip(prompts, llm.generate(prompts, max_new_tokens=new, ignore_eos=True)):
+        assert len(out) == new
+        for t, token in enumerate(out):
+            row = plain(name, prompt + out[:t])[-1]
+            assert float(row[token]) >= float(row.max()) - 3e-2 * float(row.abs().max())
+
+
+def test_the_command_line_generates(folders, plain):
+    import json
+    import os
+    import subprocess
+    import sys
+
+    from conftest import ROOT
+
+    name = "equal"
+    prompt = token_ids(CONFIGS[name]["vocab"], 9, seed=99)
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "pulse_infer"), folders[name], "--dtype", "float32",
+                          "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "6", "--greedy",
+                          "--ignore-eos", "--max-positions", "64"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    out = json.loads(run.stdout.strip().splitlines()[0])
+    assert out["output_ids"] == plain.models[name].greedy(prompt, 6)
+    # the architecture's own option is in force: a request that would pass the most positions is refused
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "pulse_infer"), folders[name], "--dtype", "float32",
+                          "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "6", "--greedy",
+                          "--ignore-eos", "--max-positions", "12"], capture_output=True, text=True, timeout=300)
+    assert run.returncode != 0 and "positions" in run.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(folders, plain, tmp_path, dtype):
+    """bin/trace_run on this architecture: steps from standard input, logits of the wanted places in files."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    from conftest import ROOT
+
+    name = "mixed"
+    vocab = CONFIGS[name]["vocab"]
+    a, b = token_ids(vocab, 70, seed=1), token_ids(vocab, 21, seed=2)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:50], "want": [0, 49]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[50:69], "want": []}, {"id": "b", "tokens": b[:20], "want": [19]}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[20:], "want": [0]}, {"id": "a", "tokens": a[69:], "want": [0]}],
+         "end": ["a", "b"]},
+    ]
+    out = tmp_path / f"out_{dtype}"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders[name], "--dtype", dtype,
+                          "--out", str(out), "--max-tokens", "192"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [line for line in run.stdout.splitlines() if line.startswith("done")] == ["done 0", "done 1", "done 2"]
+    la, lb = plain(name, a), plain(name, b)
+    read = lambda i: torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, vocab).copy())
+    close(read(0), la[[0, 49]], dtype, "step 0")
+    close(read(1), lb[[19]], dtype, "step 1")
+    close(read(2), torch.stack([lb[20], la[69]]), dtype, "step 2")
