@@ -55,10 +55,12 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     p.add_argument("--model", choices=sorted(SHAPES), default="8b", help="layer sizes: Qwen3-8B (the default), 14B or 32B")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has, if memory or time needs it")
-    p.add_argument("--workload", choices=["decode", "serving", "long-prompt"], default="decode",
+    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen"], default="decode",
                    help="decode: fixed batch at a fixed context; serving: continuous batching of requests with "
                         "seeded prompt lengths, chunked prefill mixed with decoding; long-prompt: one prompt of "
-                        "--prompt-tokens tokens in portions of --chunk tokens")
+                        "--prompt-tokens tokens in portions of --chunk tokens; dirozen: decoding and prefill of the "
+                        "Dirozen design beside Qwen3 layers of equal sizes, with both models' time by entry point")
+    p.add_argument("--compare-layers", type=int, default=4, help="dirozen: layers of the two models that are compared")
     p.add_argument("--prompt-tokens", type=int, default=16384, help="long-prompt: length of the prompt")
     p.add_argument("--requests", type=int, default=32, help="serving: number of requests")
     p.add_argument("--prompt-range", type=int, nargs=2, default=[128, 2048], help="serving: prompt lengths drawn from [lo, hi]")
@@ -221,8 +223,150 @@ def long_prompt(args, cfg, model, full_layers: int) -> int:
     return 0
 
 
+DIROZEN_SIZES = {   # layer sizes of the comparison: width, query heads, key/value heads, head size, feed-forward
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=12288),
+    "5k": dict(width=5120, heads=40, kv_heads=8, dim=128, ff=17408),
+}
+
+
+def dirozen_compare(args) -> int:
+    """Dirozen beside Qwen3 layers of equal sizes (random weights, ``--compare-layers`` layers, a vocabulary of
+    32,000): decoding at batch 1 / 8 / 32 with contexts ending at ``--context`` and a prompt of ``--prefill-tokens``
+    tokens, each through the engine's own serving loop, with the fraction of the roofline from the models' own
+    descriptions, and where an eager decoding step and a prompt step spend their time by entry point.  One JSON
+    line."""
+    import torch
+
+    from pulse_infer_amd.config import DirozenConfig, Qwen3Config
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.engine.runner import StepEntry
+    from pulse_infer_amd.models.causal_lm import expected_tensors
+    from pulse_infer_amd.models.cost import step_cost
+    from pulse_infer_amd.models.factory import build_model
+    from pulse_infer_amd.ops import timing
+    from pulse_infer_amd.sampling.params import SamplingParams
+    from pulse_infer_amd.weights.random_init import RandomSource
+
+    torch.backends.cuda.matmul.allow_tf32 = False
+    device = torch.device("cuda:0")
+    layers, vocab, page = args.compare_layers, 32000, args.page_size
+    element = 2 if args.dtype == "bfloat16" else 4
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    batches = (1, 8, 32)
+    greedy = SamplingParams(ignore_eos=True)
+
+    def configs(size):
+        qwen = Qwen3Config.from_dict(dict(
+            architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=size["width"], intermediate_size=size["ff"],
+            num_hidden_layers=layers, num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"],
+            head_dim=size["dim"], max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1e6,
+            tie_word_embeddings=False, torch_dtype="bfloat16", use_sliding_window=False), "<bench>")
+        entry = {"type": "attention",
+                 "mixer": {"dim": size["dim"], "heads": size["heads"], "kv_heads": size["kv_heads"],
+                           "q_temp": {"coef": 0.1, "every": 512}, "scale": size["dim"] ** -0.5, "vdim": size["dim"]},
+                 "mlp": {"ff": size["ff"], "kind": "dense"}}
+        dirozen = DirozenConfig.from_dict({"architecture": "Dirozen", "vocab": vocab, "width": size["width"],
+                                           "norm": {"eps": 1e-6}, "layers": [entry] * layers}, "<bench>")
+        return {"dirozen": dirozen, "qwen3": qwen}
+
+    def measure(cfg):
+        spec = cfg.model_spec()
+        source = RandomSource(expected_tensors(spec), args.seed, 0.02, torch.bfloat16, device=device)
+        model = build_model(cfg, source, mode=args.dtype, device=device)
+        pool = max(max(batches) * ((args.context + page - 1) // page + 1), (args.prefill_tokens + page - 1) // page + 1)
+        engine = ContinuousBatchEngine(model, max_batch_size=max(batches), chunk_size=512, page_size=page, num_pages=pool,
+                                       max_sequences=max(batches), max_num_batched_tokens=args.prefill_tokens,
+                                       seed=args.seed)
+        runner = engine.runner
+        for g in runner.cache.groups:
+            for t in g.spec.tensors(g.storage):
+                t.normal_(0.0, 1.0)
+        gen = torch.Generator().manual_seed(args.seed)
+        out = {}
+        steps, warmup = max(8, min(args.steps, 32)), max(4, min(args.warmup, 8))
+        for batch in batches:
+            times = []
+            start = args.context - (steps + warmup)
+            for _ in range(args.runs):
+                for _ in range(batch):
+                    rid = engine.add_request(torch.randint(0, vocab, (start + 1,), generator=gen).tolist(), steps + warmup,
+                                             greedy)
+                    engine.admit_as_computed(rid, start)
+                assert engine.run_until_complete(max_steps=warmup) == warmup
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                ran = engine.run_until_complete()
+                torch.cuda.synchronize()
+                assert ran == steps, (ran, steps)
+                times.append((time.perf_counter() - t0) / steps)
+            t = statistics.median(times)
+            cost = step_cost(spec, [(int(args.context - steps / 2.0) - 1, 1)] * batch, batch, element, element)
+            out[f"decode_b{batch}"] = {"tokens_per_s": round(batch / t, 1), "ms_per_step": round(t * 1e3, 4),
+                                       "frac_of_hbm_peak": round((cost.weight_bytes + cost.cache_bytes) / t / 1e9 / HBM_PEAK_GBS, 4)}
+        ids = torch.randint(0, vocab, (args.prefill_tokens,), generator=gen).tolist()
+        times = []
+        for r in range(args.runs + 1):
+            engine.add_request(ids, 1, greedy)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            assert engine.run_until_complete() == 1
+            torch.cuda.synchronize()
+            if r > 0:
+                times.append(time.perf_counter() - t0)
+        t = statistics.median(times)
+        flops = step_cost(spec, [(0, args.prefill_tokens)], 1, element, element).flops
+        out["prefill"] = {"tokens": args.prefill_tokens, "tokens_per_s": round(args.prefill_tokens / t, 1),
+                          "ms": round(t * 1e3, 3), "frac_of_matrix_peak": round(flops / t / peak, 4)}
+        # where the time goes, entry point by entry point: an eager decoding step of 8 requests, a prompt step
+        runner.use_graphs = False
+        names = [f"k{i}" for i in range(8)]
+        for n in names:
+            runner.add_request(n)
+            runner.reserve(n, args.context)
+            runner.cache.advance(n, args.context - 12)
+        one = lambda: runner.step([StepEntry(n, [7], [0]) for n in names])
+        for _ in range(2):
+            one()
+        with timing.record() as table:
+            for _ in range(4):
+                one()
+        out["decode_b8_us_by_entry_point"] = {k: round(ms * 1e3 / 4, 1) for k, (_, ms) in sorted(table.totals().items())}
+        for n in names:
+            runner.free_request(n)
+        for r in range(2):
+            runner.add_request("p")
+            runner.reserve("p", args.prefill_tokens)
+            if r == 0:
+                runner.step([StepEntry("p", ids, [len(ids) - 1])])
+            else:
+                with timing.record() as table:
+                    runner.step([StepEntry("p", ids, [len(ids) - 1])])
+            runner.free_request("p")
+        out["prefill_us_by_entry_point"] = {k: round(ms * 1e3, 1) for k, (_, ms) in sorted(table.totals().items())}
+        del engine, runner, model
+        torch.cuda.empty_cache()
+        return out
+
+    record = {"metric": "dirozen_beside_qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
+              "data": "synthetic", "layers": layers, "vocab": vocab, "context": args.context, "sizes": {}}
+    for name, size in DIROZEN_SIZES.items():
+        both = {model: measure(cfg) for model, cfg in configs(size).items()}
+        ratio = {k: round(both["dirozen"][k]["tokens_per_s"] / both["qwen3"][k]["tokens_per_s"], 3)
+                 for k in both["dirozen"] if "tokens_per_s" in both["dirozen"][k]}
+        record["sizes"][name] = dict(size, **both, dirozen_over_qwen3=ratio)
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
+    if args.workload == "dirozen":
+        if args.gpus != 1:
+            print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+            return 2
+        sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+        return dirozen_compare(args)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2

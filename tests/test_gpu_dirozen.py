@@ -8,9 +8,6 @@ which the serving kernels fuse the norm into the products.  Each mechanism alone
 token-by-token decoding, portions down to two tokens, mixed batches with pages used again, a far key that stands
 out, long decoding through recorded steps, and greedy generation through the scheduler.
 """
-import math
-import random
-
 import pytest
 import torch
 
@@ -503,6 +500,41 @@ def test_long_decoding_of_three_requests(runners, plain, name, dtype):
         close(torch.cat(got[k]), plain(name, ids[k])[prompt[k] - 1:], dtype, f"{name} decoding request {k}")
     if dtype == "bfloat16":
         assert runner.graph_replays > replays, "no decoding step was replayed from a recording"
+
+
+def test_a_decoding_step_runs_the_fused_kernels(runners):
+    """At the widths of a real model's layers a step of decoded tokens in bfloat16 is this package's kernels alone:
+    the attention kernel that prepares q and the key itself (no preparation launch), products that take rows not yet
+    normalised and leave the next norm's rows (the norm's kernel runs for the first layer and the last rows only), and
+    no library call; a prompt portion goes through the preparation kernel and the prompt-portion attention."""
+    from pulse_infer_amd.engine.runner import StepEntry
+    from pulse_infer_amd.ops import timing
+
+    runner = runners("wide", "bfloat16", 16, tokens=512)
+    graphs, runner.use_graphs = runner.use_graphs, False
+    try:
+        names = ["f0", "f1", "f2"]
+        for i, n in enumerate(names):
+            runner.add_request(n)
+            runner.reserve(n, 40 + i)
+        with timing.record() as prompt:
+            runner.step([StepEntry(n, token_ids(300, 30 + i, seed=i), []) for i, n in enumerate(names)])
+        with timing.record() as decode:
+            runner.step([StepEntry(n, [5 + i], [0]) for i, n in enumerate(names)])
+    finally:
+        runner.use_graphs = graphs
+        for n in names:
+            runner.free_request(n)
+    layers = len(WIDE["layers"])
+    calls = {name.split()[0]: 0 for name in decode.totals()}
+    for name, (count, _) in decode.totals().items():
+        calls[name.split()[0]] += count
+    assert calls.get("pulse_attn_decode") == layers and "pulse_qk_rope_kv" not in calls and "pulse_attn_generic" not in calls
+    assert calls.get("pulse_add_rmsnorm") == 2, calls            # the first layer's input and the wanted rows
+    assert not any(name.startswith("library") for name in calls), calls
+    assert "pulse_residual_add" not in calls and "pulse_swiglu" not in calls, calls
+    calls = {name.split()[0] for name in prompt.totals()}
+    assert {"pulse_qk_rope_kv", "pulse_attn_prefill"} <= calls and "pulse_attn_generic" not in calls, calls
 
 
 # --------------------------------------------------------------------------- generation through the scheduler
