@@ -105,7 +105,9 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
                 sq += __shfl_xor(sq, 4, 16);
                 sq += __shfl_xor(sq, 2, 16);
                 sq += __shfl_xor(sq, 1, 16);
-                if (n_in == 0 && m < M) sumsq[static_cast<int64_t>(m) * parts + n_base / 16 + tile / MT] = sq;
+                // (a slab that lies beyond N altogether, the second of a pair when N is no multiple of 32, has no part)
+                if (n_in == 0 && m < M && n_base + (tile / MT) * 16 < N)
+                    sumsq[static_cast<int64_t>(m) * parts + n_base / 16 + tile / MT] = sq;
             }
         }
     } else {

@@ -37,7 +37,8 @@ def _extras(what: str, tokens: int, nq: int, gate: Optional[torch.Tensor] = None
         return None
     ex = _Extras()
     if gate is not None:
-        _need(gate.is_cuda and gate.dtype == torch.bfloat16 and gate.dim() == 2 and gate.shape[0] == tokens
+        _gpu(what, gate)
+        _need(gate.dtype == torch.bfloat16 and gate.dim() == 2 and gate.shape[0] == tokens
               and gate.shape[1] >= nq and gate.stride(1) == 1,
               f"{what}: the gate must be bfloat16 [{tokens}, {nq}] with contiguous rows")
         ex.gate, ex.gate_stride = gate.data_ptr(), gate.stride(0) if tokens > 1 else max(nq, gate.shape[1])
