@@ -23,7 +23,7 @@ def unit_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def offset_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
-    """The layer norm: unit_rms(x) * (1 + w), the weight being stored around zero."""
+    """The layer norm: unit_rms(x) * (1 + w), the weight being stored as its distance from one."""
     return unit_rms(x, eps) * (1.0 + w)
 
 

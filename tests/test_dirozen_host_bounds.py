@@ -1,4 +1,4 @@
-"""The host side of whole steps on the CPU, with every HIP entry point replaced by a checker of its operands.
+"""The host side of whole steps on the CPU, with every HIP entry point replaced by a function that verifies its operands.
 
 Seeded random Dirozen configurations (the sweep of tests/test_gpu_dirozen.py: head sizes the matrix-core kernels take
 and two they do not, widths that are no multiple of 16, one query head, up to four cache groups) run whole prompts,
@@ -131,12 +131,12 @@ def check(name, args):
         h, delta, _, parts, n, _ = args
         need(room(h) >= val(n) and room(delta) >= val(parts) * val(n), "operands")
     elif name != "pulse_attn_plan":
-        raise AssertionError(f"an entry point without a checker: {name}")
+        raise AssertionError(f"an entry point that nothing verifies: {name}")
 
 
 @pytest.fixture
 def checked_kernels(monkeypatch):
-    """Every entry point becomes its checker; pointers remember their tensors; library products run on the CPU."""
+    """Every entry point becomes the function that verifies its operands; pointers remember their tensors; library products run on the CPU."""
     from pulse_infer_amd.engine import runner as runner_module
     from pulse_infer_amd.ops import attention_mfma, kernels
 

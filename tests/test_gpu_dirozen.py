@@ -105,7 +105,7 @@ def tol(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hidden", [96, 1000, 2048])
-def test_norm_with_a_weight_stored_around_zero(dtype, hidden):
+def test_norm_with_a_weight_stored_as_its_distance_from_one(dtype, hidden):
     """x / sqrt(mean(x^2) + eps) * (1 + w): the one is added in float32, so a weight of 2^-9, which bfloat16 cannot
     add to one, still shows."""
     from pulse_infer_amd.ops import kernels
@@ -299,7 +299,7 @@ def test_decoded_tokens_from_the_raw_projection(case, split):
 
 def test_rows_for_the_next_norm_carry_one_plus_the_weight():
     """The few-rows product that adds into the residual leaves the new rows once more, multiplied by the next norm's
-    factors: for a weight stored around zero these are 1 + w, the one added in float32."""
+    factors: for a weight stored as its distance from one these are 1 + w, the one added in float32."""
     from pulse_infer_amd.ops import kernels
 
     m, n, kk = 5, 1024, 2048
