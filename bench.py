@@ -61,6 +61,7 @@ def parse_args() -> argparse.Namespace:
                         "--prompt-tokens tokens in portions of --chunk tokens; dirozen: decoding and prefill of the "
                         "Dirozen design beside Qwen3 layers of equal sizes, with both models' time by entry point")
     p.add_argument("--compare-layers", type=int, default=4, help="dirozen: layers of the two models that are compared")
+    p.add_argument("--compare-sizes", default="2k,4k,5k", help="dirozen: which of the layer sizes 2k, 4k, 5k (widths) to run")
     p.add_argument("--prompt-tokens", type=int, default=16384, help="long-prompt: length of the prompt")
     p.add_argument("--requests", type=int, default=32, help="serving: number of requests")
     p.add_argument("--prompt-range", type=int, nargs=2, default=[128, 2048], help="serving: prompt lengths drawn from [lo, hi]")
@@ -288,7 +289,7 @@ def dirozen_compare(args) -> int:
         for batch in batches:
             times = []
             start = args.context - (steps + warmup)
-            for _ in range(args.runs):
+            for r in range(args.runs + 1):       # the first run warms up (kernels loaded, the step recorded)
                 for _ in range(batch):
                     rid = engine.add_request(torch.randint(0, vocab, (start + 1,), generator=gen).tolist(), steps + warmup,
                                              greedy)
@@ -299,20 +300,21 @@ def dirozen_compare(args) -> int:
                 ran = engine.run_until_complete()
                 torch.cuda.synchronize()
                 assert ran == steps, (ran, steps)
-                times.append((time.perf_counter() - t0) / steps)
+                if r > 0:
+                    times.append((time.perf_counter() - t0) / steps)
             t = statistics.median(times)
             cost = step_cost(spec, [(int(args.context - steps / 2.0) - 1, 1)] * batch, batch, element, element)
             out[f"decode_b{batch}"] = {"tokens_per_s": round(batch / t, 1), "ms_per_step": round(t * 1e3, 4),
                                        "frac_of_hbm_peak": round((cost.weight_bytes + cost.cache_bytes) / t / 1e9 / HBM_PEAK_GBS, 4)}
         ids = torch.randint(0, vocab, (args.prefill_tokens,), generator=gen).tolist()
         times = []
-        for r in range(args.runs + 1):
+        for r in range(args.runs + 2):           # two warm-up runs: the vendor library chooses its kernels in the first
             engine.add_request(ids, 1, greedy)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             assert engine.run_until_complete() == 1
             torch.cuda.synchronize()
-            if r > 0:
+            if r > 1:
                 times.append(time.perf_counter() - t0)
         t = statistics.median(times)
         flops = step_cost(spec, [(0, args.prefill_tokens)], 1, element, element).flops
@@ -351,6 +353,8 @@ def dirozen_compare(args) -> int:
     record = {"metric": "dirozen_beside_qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
               "data": "synthetic", "layers": layers, "vocab": vocab, "context": args.context, "sizes": {}}
     for name, size in DIROZEN_SIZES.items():
+        if name not in args.compare_sizes.split(","):
+            continue
         both = {model: measure(cfg) for model, cfg in configs(size).items()}
         ratio = {k: round(both["dirozen"][k]["tokens_per_s"] / both["qwen3"][k]["tokens_per_s"], 3)
                  for k in both["dirozen"] if "tokens_per_s" in both["dirozen"][k]}
