@@ -113,7 +113,7 @@ class DirozenConfig(ModelConfig):
                                   f"(known: {', '.join(MLP_KINDS)})")
             ff = f.integer("ff")
         return DirozenLayer(type=kind, heads=m.integer("heads"), kv_heads=m.integer("kv_heads"), dim=m.integer("dim"),
-                            vdim=m.integer("vdim"), scale=m.number("scale"), temp_coef=t.number("coef"),
+                            vdim=m.integer("vdim", m.integer("dim")), scale=m.number("scale"), temp_coef=t.number("coef"),
                             temp_every=t.integer("every"), ff=ff)
 
     # --------------------------------------------------------------- validation
