@@ -97,6 +97,12 @@ class Linear:
                     and out.stride(0) % 8 == 0 and out.data_ptr() % 16 == 0:
                 kernels.gemm_tile(x, w, out)
                 return out
+            if not self.rows_aligned(x, w):
+                # The vendor library is handed only operands whose rows keep 16-byte alignment (inner sizes that are
+                # multiples of 8, which every shape of a real model is); anything else goes through this package's
+                # fused-multiply-add product, which takes any shape and guards every access.
+                kernels.gemm_f32(x, w, out)
+                return out
             global library_calls
             library_calls += 1
             if out.dtype == torch.bfloat16:
@@ -205,6 +211,12 @@ class Linear:
         while splits > 1 and (self.in_features % splits or (self.in_features // splits) % 64):
             splits //= 2
         return splits if splits > 1 else 0
+
+    @staticmethod
+    def rows_aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
+        """Whether the rows of both bfloat16 operands start at multiples of 16 bytes."""
+        return (x.shape[1] % 8 == 0 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0)
+                and (w.shape[0] <= 1 or w.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
     def operands_ok(self, x: torch.Tensor) -> bool:
         """Contiguous, aligned bfloat16 rows of a length the kernels' 16-byte loads take."""

@@ -317,6 +317,27 @@ def test_rows_for_the_next_norm_carry_one_plus_the_weight():
     assert torch.allclose(sums.sum(1).cpu().to(F64), (new * new).sum(1), rtol=1e-3)
 
 
+@pytest.mark.parametrize("rows", [3, 40, 333])
+def test_products_with_unaligned_rows_stay_off_the_vendor_library(rows):
+    """An inner size that is no multiple of 8 (heads of 20 channels, say) leaves bfloat16 rows off 16-byte alignment:
+    such a product runs on this package's guarded multiply-add kernel, in any number of rows, into bfloat16 and into
+    float32."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.parts import linear
+
+    n, kk = 200, 300
+    w, wref = stored(rnd(n, kk, seed=1, scale=kk ** -0.5), torch.bfloat16)
+    x, xref = stored(rnd(rows, kk, seed=2), torch.bfloat16)
+    product = linear.Linear(w, "bfloat16")
+    before = linear.library_calls
+    for dtype in (torch.bfloat16, torch.float32):
+        out = torch.full((rows, n), float("nan"), dtype=dtype, device=DEV)
+        product.forward(x, out)
+        assert torch.allclose(out.cpu().to(F64), xref @ wref.T, **tol(dtype))
+    assert linear.library_calls == before
+
+
 # ------------------------------------------------------------------------------------------------ whole models
 LENGTH = {"mixed": 150, "equal": 170, "wide": 90}
 
