@@ -163,9 +163,23 @@ ATTENTION_CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", ATTENTION_CASES)
-@pytest.mark.parametrize("path", ["generic", "matrix", "matrix_splits", "portion", "portion_splits"])
+def attention_paths():
+    """(case, kernel path, storage type) for every combination that exists: the generic kernel takes everything, the
+    matrix-core kernels bfloat16 with head sizes in steps of 16 and pages of 16 and more, the prompt-portion kernel
+    has splits for head sizes 32, 64 and 128."""
+    out = []
+    for case in ATTENTION_CASES:
+        for dtype in (torch.float32, torch.bfloat16):
+            out.append((case, "generic", dtype))
+        if case["d"] % 16 == 0 and case["bs"] % 16 == 0:
+            for path in ("matrix", "matrix_splits", "portion"):
+                out.append((case, path, torch.bfloat16))
+            if case["d"] in (32, 64, 128):
+                out.append((case, "portion_splits", torch.bfloat16))
+    return out
+
+
+@pytest.mark.parametrize("case,path,dtype", attention_paths())
 def test_attention_with_keys_as_values_temperature_and_gate(case, path, dtype):
     """One step of a portion of request 0 beside single tokens of the others, over pages that hold the earlier
     tokens: the preparation kernel (norm without weights, temperature by position, the raw key as the value) and each
@@ -174,10 +188,8 @@ def test_attention_with_keys_as_values_temperature_and_gate(case, path, dtype):
     from pulse_infer_amd.ops import kernels
 
     nq, nkv, d, bs, lens, portion, every = (case[x] for x in ("nq", "nkv", "d", "bs", "lens", "portion", "every"))
-    if path != "generic" and (dtype != torch.bfloat16 or not M.supported(d, bs, dtype, dtype)):
-        pytest.skip("the matrix-core kernels take bfloat16, head sizes in steps of 16 and pages of 16 and more")
-    if path == "portion_splits" and d not in M.PREFILL_SPLIT_HEAD_DIMS:
-        pytest.skip("this head size's portion kernel has no splits")
+    assert path == "generic" or M.supported(d, bs, dtype, dtype)
+    assert path != "portion_splits" or d in M.PREFILL_SPLIT_HEAD_DIMS
     eps, coef, scale, share = 1e-5, 0.35, 0.21, nq // nkv
     kc, vc, table = paged(lens, nkv, d, bs, dtype, seed=3)
     gate_rows = 16
