@@ -25,7 +25,7 @@ from dataclasses import dataclass, field
 from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 from .page_pool import OutOfPages, PageError, PagePool
-from .specs import PagedKVSpec, StateSpec, check_spec  # noqa: F401  (the two specs are part of this module's names)
+from .specs import CombinedSpec, PagedKVSpec, StateSpec, check_spec, members  # noqa: F401  (the specs are part of this module's names)
 
 
 class CacheError(RuntimeError):
@@ -107,27 +107,31 @@ class CacheManager:
         self.page_size = int(page_size)
         self.run_specs = list(run_specs)
         self.groups: List[CacheGroup] = []
-        self.run_group: Dict[int, Tuple[int, int]] = {}   # run -> (group, index within group)
-        self.state_runs: Dict[int, Any] = {}
+        # Keys of the two maps below: the run's number, or (run, member) for a member of a run's combined spec.
+        self.run_group: Dict[Any, Tuple[int, int]] = {}   # -> (group, index within group)
+        self.state_runs: Dict[Any, Any] = {}
         by_spec: Dict[Any, CacheGroup] = {}
-        for run, spec in enumerate(self.run_specs):
-            if spec is None:
+        for run, whole in enumerate(self.run_specs):
+            if whole is None:
                 continue
-            check_spec(spec, run)
-            if spec.per_token:
-                group = by_spec.get(spec)
-                if group is None:
-                    pages = (group_pages or {}).get(spec, num_pages)
-                    group = CacheGroup(len(self.groups), spec, self.page_size, [], PagePool(pages))
-                    by_spec[spec] = group
-                    self.groups.append(group)
-                self.run_group[run] = (group.index, len(group.runs))
-                group.runs.append(run)
-            else:
-                self.state_runs[run] = spec
+            check_spec(whole, run)
+            parts = members(whole)
+            units = [(run, whole)] if parts is None else [((run, j), part) for j, part in enumerate(parts)]
+            for key, spec in units:
+                if spec.per_token:
+                    group = by_spec.get(spec)
+                    if group is None:
+                        pages = (group_pages or {}).get(spec, num_pages)
+                        group = CacheGroup(len(self.groups), spec, self.page_size, [], PagePool(pages))
+                        by_spec[spec] = group
+                        self.groups.append(group)
+                    self.run_group[key] = (group.index, len(group.runs))
+                    group.runs.append(key)
+                else:
+                    self.state_runs[key] = spec
         self.slots = StateSlots(max_requests)
         self.requests: Dict[Hashable, _Request] = {}
-        self.state: Dict[int, object] = {}  # run -> [slots, *shape] array
+        self.state: Dict[Any, object] = {}  # run (or (run, member)) -> [slots, *shape] array
         self.max_requests = int(max_requests)
         self._clock = 0     # source of the requests' stamps
 
@@ -148,11 +152,17 @@ class CacheManager:
         spec = self.run_specs[run]
         if spec is None:
             return None
+        parts = members(spec)
+        if parts is not None:
+            return tuple(self._view_of((run, j), part, writable) for j, part in enumerate(parts))
+        return self._view_of(run, spec, writable)
+
+    def _view_of(self, key: Any, spec: Any, writable: bool) -> Any:
         if spec.per_token:
-            g, i = self.run_group[run]
+            g, i = self.run_group[key]
             group = self.groups[g]
             return spec.view(group.storage, i, g, group.page_size, writable)
-        return spec.view(self.state[run], 0, -1, self.page_size, writable)
+        return spec.view(self.state[key], 0, -1, self.page_size, writable)
 
     def storage_bytes(self, element_size: int) -> int:
         return sum(len(g.runs) * g.pool.num_pages * g.page_size * g.spec.bytes_per_token(element_size)

@@ -19,6 +19,11 @@ A spec is a small hashable object that the cache manager asks, never inspects:
   needs to address it (``group`` is the key into ``StepContext.block_tables``).
 * ``tensors(storage)`` — the storage's tensors, for whoever counts or fills them.
 
+A run whose mixer keeps several things (pages of one branch and a state of
+another, say) answers with a ``CombinedSpec`` of their specs; each of them is
+then served as if it were a run's own, and the run is handed the tuple of
+their views.
+
 Two specs are provided: keys and values of attention heads in pages, and a plain
 array per request.  A mixer that pages something else per token (one row of some
 width, keys and values of different widths, the tail of a convolution) brings a
@@ -102,8 +107,30 @@ class StateSpec:
         return [storage]
 
 
+@dataclass(frozen=True)
+class CombinedSpec:
+    """What a run keeps when it keeps several things: the specs of each, in the order in which the run's mixer expects
+    their views (a tuple, one view a spec).  The members are ordinary specs: per-token ones join the groups of equal
+    specs, the others get arrays by slot."""
+
+    parts: Tuple[Any, ...]
+
+
+def members(spec: Any) -> Optional[Tuple[Any, ...]]:
+    """The specs a ``CombinedSpec`` holds; None for a plain spec."""
+    return tuple(spec.parts) if isinstance(spec, CombinedSpec) else None
+
+
 def check_spec(spec: Any, run: int) -> None:
     """A clear error for something that is no cache spec."""
+    if isinstance(spec, CombinedSpec):
+        if not spec.parts:
+            raise TypeError(f"run {run}: a combined cache spec needs at least one member")
+        for part in spec.parts:
+            if isinstance(part, CombinedSpec):
+                raise TypeError(f"run {run}: combined cache specs do not nest")
+            check_spec(part, run)
+        return
     if not isinstance(getattr(spec, "per_token", None), bool) or not all(
             callable(getattr(spec, name, None)) for name in ("allocate", "view", "tensors")):
         raise TypeError(f"run {run}: {spec!r} is no cache spec (it needs per_token, allocate, view and tensors; "

@@ -13,7 +13,7 @@
 // (reference: src/ops/kernels/cuda/embedding_kernel.cu:7-28 leaves zeros silently)
 template <typename TW>
 __global__ void embed_gather_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
-                                    float* __restrict__ out, int hidden, int vocab, int* bad_id) {
+                                    float* __restrict__ out, int hidden, int vocab, int* bad_id, float scale) {
     const int t = blockIdx.x;
     const int id = ids[t];
     float* dst = out + static_cast<int64_t>(t) * hidden;
@@ -23,18 +23,18 @@ __global__ void embed_gather_kernel(const int* __restrict__ ids, const TW* __res
         return;
     }
     const TW* src = table + static_cast<int64_t>(id) * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32<TW>(src[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32<TW>(src[i]) * scale;
 }
 
 extern "C" int pulse_embed_gather(const int* ids, const void* table, int table_dtype, float* out,
-                                  int tokens, int hidden, int vocab, int* bad_id, hipStream_t stream) {
+                                  int tokens, int hidden, int vocab, int* bad_id, float scale, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes T=%d H=%d V=%d", tokens, hidden, vocab);
     PULSE_REQUIRE(pulse_dtype_ok(table_dtype), "embed_gather: bad dtype tag %d", table_dtype);
     PULSE_REQUIRE(ids && table && out && bad_id, "embed_gather: null pointer");
     if (tokens == 0) return 0;
     PULSE_DISPATCH_DTYPE(table_dtype, TW,
         hipLaunchKernelGGL(embed_gather_kernel<TW>, dim3(tokens), dim3(256), 0, stream, ids,
-                           static_cast<const TW*>(table), out, hidden, vocab, bad_id));
+                           static_cast<const TW*>(table), out, hidden, vocab, bad_id, scale));
     PULSE_LAUNCH_CHECK("embed_gather");
     return 0;
 }

@@ -69,8 +69,9 @@ def _int_vec(what: str, t: torch.Tensor, n: Optional[int] = None) -> None:
 
 
 # ---------------------------------------------------------------------------
-def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_id: torch.Tensor) -> None:
-    """out[t] = float32(table[ids[t]]); ``bad_id`` (int32[1]) is raised for an id outside the table."""
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_id: torch.Tensor,
+                 scale: float = 1.0) -> None:
+    """out[t] = float32(table[ids[t]]) * scale; ``bad_id`` (int32[1]) is raised for an id outside the table."""
     _gpu("embed_gather", ids, table, out, bad_id)
     tokens = ids.numel()
     vocab, hidden = table.shape
@@ -80,7 +81,7 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_
           f"embed_gather: out must be float32 [{tokens}, {hidden}], got {out.dtype} {tuple(out.shape)}")
     _need(bad_id.dtype == torch.int32 and bad_id.numel() >= 1, "embed_gather: bad_id must be int32[1]")
     call("pulse_embed_gather", _ptr(ids), _ptr(table), _i32(_tag(table, "embed_gather")), _ptr(out),
-         _i32(tokens), _i32(hidden), _i32(vocab), _ptr(bad_id), _stream())
+         _i32(tokens), _i32(hidden), _i32(vocab), _ptr(bad_id), _f32(scale), _stream())
 
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
@@ -595,3 +596,224 @@ def mark_seen(masks: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, voc
     _int_vec("mark_seen: tokens", tokens, rows.numel())
     call("pulse_mark_seen", _ptr(masks), _i32(masks.shape[1]), _ptr(rows), _ptr(tokens), _i32(rows.numel()),
          _i32(vocab), _stream())
+
+
+# ---------------------------------------------------------------------------
+# A layer whose norm comes after the sum; small element-wise kernels
+ACTIVATIONS = {"relu2": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def scale_add_rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, alpha: float = 1.0,
+                      delta: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None,
+                      column_scale: Optional[torch.Tensor] = None, copy: Optional[torch.Tensor] = None) -> None:
+    """h <- rmsnorm(alpha * h + column_scale * (delta + delta2)) * weight, float32 in place; ``copy`` receives the new
+    rows once more, rounded to its storage type.  The updates may be of any of the two storage types."""
+    _gpu("scale_add_rmsnorm", h, weight, delta, delta2, column_scale, copy)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "scale_add_rmsnorm: h must be contiguous float32 [T, H]")
+    rows, hidden = h.shape
+    for d in (delta, delta2, copy):
+        _need(d is None or (tuple(d.shape) == (rows, hidden) and d.is_contiguous()),
+              f"scale_add_rmsnorm: updates and the copy must be contiguous [{rows}, {hidden}]")
+    _need(delta is not None or delta2 is None, "scale_add_rmsnorm: a second update without a first")
+    _need(weight.numel() == hidden and weight.is_contiguous(), f"scale_add_rmsnorm: weight must hold {hidden} values")
+    _need(column_scale is None or (column_scale.numel() == hidden and column_scale.is_contiguous()
+                                   and column_scale.dtype == weight.dtype),
+          f"scale_add_rmsnorm: the column factors must hold {hidden} values of the weight's storage type")
+    tag = lambda t: _tag(t, "scale_add_rmsnorm") if t is not None else 0
+    call("pulse_scale_add_rmsnorm", _ptr(h), _ptr(delta), _i32(tag(delta)), _ptr(delta2), _i32(tag(delta2)),
+         _ptr(column_scale), _ptr(weight), _i32(tag(weight)), _ptr(copy), _i32(tag(copy)), _i32(rows), _i32(hidden),
+         _f32(alpha), _f32(eps), _stream())
+
+
+def activation(x: torch.Tensor, out: torch.Tensor, kind: str) -> None:
+    """out = act(x) element by element: ``relu2`` (the square of relu), ``gelu_tanh``, ``silu``."""
+    _gpu("activation", x, out)
+    _need(kind in ACTIVATIONS, f"activation: unknown activation '{kind}' (known: {sorted(ACTIVATIONS)})")
+    _need(x.shape == out.shape and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous(),
+          "activation: contiguous tensors of one shape and storage type are needed")
+    call("pulse_activation", _ptr(x), _ptr(out), _i32(_tag(x, "activation")), _i64(x.numel()), _i32(ACTIVATIONS[kind]),
+         _stream())
+
+
+def softcap(x: torch.Tensor, cap: float) -> None:
+    """x <- cap * tanh(x / cap), in place on float32."""
+    _gpu("softcap", x)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and cap > 0, "softcap: a contiguous float32 tensor and a positive cap")
+    call("pulse_softcap", _ptr(x), _i64(x.numel()), _f32(cap), _stream())
+
+
+def round_rows(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = x (float32) in out's storage type."""
+    _gpu("round_rows", x, out)
+    _need(x.dtype == torch.float32 and x.shape == out.shape and x.is_contiguous() and out.is_contiguous(),
+          "round_rows: a contiguous float32 tensor and a contiguous result of its shape")
+    call("pulse_round_rows", _ptr(x), _ptr(out), _i32(_tag(out, "round_rows")), _i64(x.numel()), _stream())
+
+
+# ---------------------------------------------------------------------------
+# Attention inputs with a norm over the whole projection, biases, and keys and values of different widths
+def qkv_rows(qkv: torch.Tensor, q_out: torch.Tensor, nq: int, nkv: int, d: int, dv: int, stored: int,
+             biases: Optional[tuple], norm_weights: Optional[tuple], eps: float, cos: Optional[torch.Tensor],
+             sin: Optional[torch.Tensor], rotary_dim: int, pairing: int, kcache: Optional[torch.Tensor],
+             vcache: Optional[torch.Tensor], positions: torch.Tensor, token_entry: torch.Tensor,
+             block_table: Optional[torch.Tensor], write_kv: bool = True, value_scale: float = 1.0,
+             norm: bool = True) -> None:
+    """q, k, v of ``qkv`` [T, nq*d + nkv*d + nkv*dv] -> biased, q and k normed over the whole row (``norm``, with
+    ``norm_weights`` = (wq [nq*d], wk [nkv*d]) or None), rotated; q to ``q_out`` [T, nq*stored], k and v (times
+    ``value_scale``) to their pages, every head filled with zeros up to ``stored`` channels."""
+    _gpu("qkv_rows", qkv, q_out, cos, sin, kcache, vcache, positions, token_entry, block_table)
+    tokens = qkv.shape[0]
+    cols = nq * d + (nkv * (d + dv) if write_kv else 0)
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= cols, f"qkv_rows: qkv needs {cols} contiguous columns")
+    _need(q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == tokens and q_out.shape[1] >= nq * stored
+          and q_out.dtype == qkv.dtype, f"qkv_rows: q_out must be [{tokens}, {nq * stored}] of qkv's storage type")
+    _int_vec("qkv_rows: positions", positions, tokens)
+    _int_vec("qkv_rows: token_entry", token_entry, tokens)
+    w_tag = None
+    ptrs = [None] * 5
+    sizes = (nq * d, nkv * d, nkv * dv, nq * d, nkv * d)
+    given = list(biases or (None, None, None)) + list(norm_weights or (None, None))
+    for i, (t, n) in enumerate(zip(given, sizes)):
+        if t is None:
+            continue
+        _gpu("qkv_rows", t)
+        _need(t.numel() == n and t.is_contiguous(), f"qkv_rows: a bias or norm weight must hold {n} values")
+        tag = _tag(t, "qkv_rows")
+        _need(w_tag is None or w_tag == tag, "qkv_rows: biases and norm weights must be of one storage type")
+        w_tag = tag
+        ptrs[i] = t
+    if cos is not None:
+        half = rotary_dim // 2
+        for t in (cos, sin):
+            _need(t is not None and t.dtype == torch.float32 and t.is_contiguous() and t.shape[0] >= tokens
+                  and t.shape[1] == half, f"qkv_rows: cos/sin must be float32 [T, {half}]")
+    pages = page_size = width = 0
+    c_tag = 0
+    if write_kv:
+        _need(kcache is not None and vcache is not None and block_table is not None, "qkv_rows: the cache is missing")
+        pages, page_size = _check_cache("qkv_rows", kcache, vcache, nkv, stored)
+        _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+              "qkv_rows: block_table must be contiguous int32 [entries, width]")
+        width = block_table.shape[1]
+        c_tag = _tag(kcache, "qkv_rows")
+    call("pulse_qkv_rows", _ptr(qkv), _i32(_tag(qkv, "qkv_rows")), _i64(qkv.stride(0)), _ptr(ptrs[0]), _ptr(ptrs[1]),
+         _ptr(ptrs[2]), _ptr(ptrs[3]), _ptr(ptrs[4]), _i32(w_tag or 0), _i32(1 if norm else 0), _f32(eps), _ptr(cos),
+         _ptr(sin), _i32(rotary_dim if cos is not None else 0), _i32(pairing), _ptr(q_out), _i64(q_out.stride(0)),
+         _ptr(kcache if write_kv else None), _ptr(vcache if write_kv else None), _i32(c_tag), _ptr(positions),
+         _ptr(token_entry), _ptr(block_table if write_kv else None), _i32(width), _i32(tokens), _i32(nq), _i32(nkv),
+         _i32(d), _i32(dv), _i32(stored), _i32(page_size), _i32(pages), _i32(1 if write_kv else 0), _f32(value_scale),
+         _stream())
+
+
+# ---------------------------------------------------------------------------
+# Linear attention with a decay per head
+def lightning_row_groups(entries: int, heads: int, d: int, dv: int) -> int:
+    """Over how many lanes ``lightning_scan`` shares a column's rows out: the fewest (1, 4, 16) that give the launch
+    about as many wavefronts as the chip has places for."""
+    from .device import compute_units
+    want = 4 * compute_units()
+    for r in (1, 4, 16):
+        if r == 16 and d <= 32:
+            break
+        if entries * heads * ((dv * r + 63) // 64) >= want:
+            return r
+    return 16 if d > 32 else 4
+
+
+def lightning_scan(x: torch.Tensor, q0: int, k0: int, v0: int, out: torch.Tensor, state: torch.Tensor,
+                   decay: torch.Tensor, entry_first_row: torch.Tensor, entry_start: torch.Tensor,
+                   entry_slot: torch.Tensor, heads: int, d: int, dv: int, activation: str = "silu",
+                   row_groups: int = 1) -> None:
+    """For every entry of the step, token by token: S <- decay_h S + k v^T, out = S^T q, per head, in float32;
+    S [slots, heads, d, dv] is the state of the entry's slot, zero when the entry starts at position 0."""
+    _gpu("lightning_scan", x, out, state, decay, entry_first_row, entry_start, entry_slot)
+    entries = entry_start.numel()
+    _need(x.dim() == 2 and x.stride(1) == 1, "lightning_scan: x must be a matrix with contiguous rows")
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == x.shape[0]
+          and out.shape[1] >= heads * dv, f"lightning_scan: out must be float32 [{x.shape[0]}, {heads * dv}]")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 4
+          and tuple(state.shape[1:]) == (heads, d, dv), f"lightning_scan: state must be float32 [slots, {heads}, {d}, {dv}]")
+    _need(decay.dtype == torch.float32 and decay.is_contiguous() and decay.numel() == heads,
+          f"lightning_scan: decay must hold {heads} float32 values")
+    _int_vec("lightning_scan: entry_first_row", entry_first_row, entries + 1)
+    _int_vec("lightning_scan: entry_start", entry_start, entries)
+    _int_vec("lightning_scan: entry_slot", entry_slot, entries)
+    _need(activation in ("none", "silu"), "lightning_scan: the activation is 'none' or 'silu'")
+    width = x.shape[1]
+    _need(min(q0, k0, v0) >= 0 and max(q0, k0) + heads * d <= width and v0 + heads * dv <= width,
+          "lightning_scan: q, k or v columns lie outside x")
+    call("pulse_lightning_scan", _ptr(x), _i32(_tag(x, "lightning_scan")), _i64(x.stride(0)), _i32(q0), _i32(k0), _i32(v0),
+         _ptr(out), _i64(out.stride(0)), _ptr(state), _i32(state.shape[0]), _ptr(decay), _ptr(entry_first_row),
+         _ptr(entry_start), _ptr(entry_slot), _i32(entries), _i32(heads), _i32(d), _i32(dv),
+         _i32(1 if activation == "silu" else 0), _i32(row_groups), _stream())
+
+
+def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, eps: float,
+                  scale: float = 1.0) -> None:
+    """out = scale * o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate) row by row; o float32, gate and out (rows may
+    be strided) of one storage type."""
+    _gpu("gated_rmsnorm", o, weight, gate, out)
+    tokens, n = o.shape
+    _need(o.dtype == torch.float32 and o.stride(1) == 1, "gated_rmsnorm: o must be float32 with contiguous rows")
+    _need(out.dim() == 2 and out.shape[0] == tokens and out.shape[1] == n and out.stride(1) == 1,
+          f"gated_rmsnorm: out must be [{tokens}, {n}] with contiguous rows")
+    _need(gate is None or (gate.shape == out.shape and gate.stride(1) == 1 and gate.dtype == out.dtype),
+          "gated_rmsnorm: the gate must have out's shape and storage type")
+    _need(weight.numel() == n and weight.is_contiguous(), f"gated_rmsnorm: weight must hold {n} values")
+    row = lambda t: t.stride(0) if tokens > 1 else max(n, t.shape[1])
+    call("pulse_gated_rmsnorm", _ptr(o), _i64(row(o)), _ptr(weight), _i32(_tag(weight, "gated_rmsnorm")), _ptr(gate),
+         _i64(row(gate) if gate is not None else 0), _ptr(out), _i64(row(out)), _i32(_tag(out, "gated_rmsnorm")),
+         _i32(tokens), _i32(n), _f32(eps), _f32(scale), _stream())
+
+
+# ---------------------------------------------------------------------------
+# Routed feed-forward
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
+              weight: torch.Tensor) -> None:
+    """Softmax over a row of router logits, the ``top`` outputs with the largest score + correction, and their scores
+    divided by their sum: idx int32 [T, top], weight float32 [T, top]."""
+    _gpu("moe_route", logits, correction, idx, weight)
+    tokens, n = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "moe_route: logits must be contiguous float32")
+    _need(correction is None or (correction.numel() == n and correction.is_contiguous()),
+          f"moe_route: the correction must hold {n} values")
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and tuple(idx.shape) == (tokens, top)
+          and weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == (tokens, top),
+          f"moe_route: idx int32 and weight float32 must be [{tokens}, {top}]")
+    call("pulse_moe_route", _ptr(logits), _ptr(correction), _i32(_tag(correction, "moe_route") if correction is not None else 0),
+         _ptr(idx), _ptr(weight), _i32(tokens), _i32(n), _i32(top), _stream())
+
+
+def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor) -> None:
+    """act[(t, k)] = silu(gate_e x_t) * (up_e x_t) for e = idx[t, k] < experts; rows of identity experts are left alone."""
+    _gpu("moe_gate_up", x, w_gate, w_up, idx, act)
+    tokens, hidden = x.shape
+    experts, ff, h2 = w_gate.shape
+    top = idx.shape[1]
+    _need(h2 == hidden and w_up.shape == w_gate.shape and w_gate.is_contiguous() and w_up.is_contiguous()
+          and w_gate.dtype == w_up.dtype, "moe_gate_up: stacked weights [experts, ff, hidden] of one storage type")
+    _need(x.is_contiguous() and act.is_contiguous() and act.dtype == x.dtype and tuple(act.shape) == (tokens * top, ff),
+          f"moe_gate_up: act must be [{tokens * top}, {ff}] of x's storage type")
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and idx.shape[0] == tokens, "moe_gate_up: idx must be int32 [T, top]")
+    call("pulse_moe_gate_up", _ptr(x), _i32(_tag(x, "moe_gate_up")), _ptr(w_gate), _ptr(w_up),
+         _i32(_tag(w_gate, "moe_gate_up")), _ptr(idx), _ptr(act), _i32(tokens), _i32(hidden), _i32(ff), _i32(experts),
+         _i32(top), _stream())
+
+
+def moe_down(x: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor, weight: torch.Tensor,
+             out: torch.Tensor) -> None:
+    """out[t] = sum_k weight[t, k] * (down_e act[(t, k)] if e = idx[t, k] < experts else x[t]), float32."""
+    _gpu("moe_down", x, act, w_down, idx, weight, out)
+    tokens, hidden = x.shape
+    experts, h2, ff = w_down.shape
+    top = idx.shape[1]
+    _need(h2 == hidden and w_down.is_contiguous(), "moe_down: the stacked weight must be [experts, hidden, ff]")
+    _need(x.is_contiguous() and act.is_contiguous() and act.dtype == x.dtype and tuple(act.shape) == (tokens * top, ff),
+          f"moe_down: act must be [{tokens * top}, {ff}] of x's storage type")
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and tuple(idx.shape) == (tokens, top)
+          and weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == (tokens, top),
+          "moe_down: idx int32 and weight float32 must be [T, top]")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (tokens, hidden),
+          f"moe_down: out must be float32 [{tokens}, {hidden}]")
+    call("pulse_moe_down", _ptr(x), _ptr(act), _i32(_tag(x, "moe_down")), _ptr(w_down), _i32(_tag(w_down, "moe_down")),
+         _ptr(idx), _ptr(weight), _ptr(out), _i32(tokens), _i32(hidden), _i32(ff), _i32(experts), _i32(top), _stream())

@@ -1,0 +1,158 @@
+"""Attention over a paged cache whose inputs are prepared a row at a time: biases on the projections, a norm of q
+and of k over a token's WHOLE projection (all heads together, a weight per channel of the projection), keys and values
+of different widths.  Window, grouped key/value heads, rotation on the first channels of every head and the scale are
+those of ``attention``; so are the attention kernels, which this part inherits.
+
+Parameters beyond those of ``attention``: ``value_dim`` (default ``head_dim``); ``bias`` (q, k and v have biases,
+named by ``names`` as ``q_bias`` ...); ``qk_norm``: "projection" or False; ``qk_norm_eps``; ``out_scale`` (a factor on
+the result; it is multiplied into the values as they are stored, in float32 before their one rounding).
+
+Keys and values are stored with one width D = max(head_dim, value_dim) rounded up to a multiple of 16, the missing
+channels as zeros: zero key channels add nothing to a score, and zero value channels come out as zeros, which meet
+zero columns of the output weight.  The attention kernels then see ordinary heads of D channels.
+
+It answers the protocol of a branch of ``side_by_side`` (``inner_width``, ``out_weight()``, ``forward_inner``).
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, Optional
+
+import torch
+
+from ..cache.manager import PagedKVSpec
+from ..ops import kernels
+from ..weights.store import TensorSpec
+from .attention import PagedAttention
+from .base import MIXERS, BuildContext, PagedCacheView, Part, StepContext, StepCost, joined
+from .linear import Linear
+
+
+def stored_width(d: int, dv: int) -> int:
+    return (max(d, dv) + 15) // 16 * 16
+
+
+@MIXERS.register("attention_rows")
+class RowPreparedAttention(PagedAttention):
+    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_bias": "q.b", "k_bias": "k.b", "v_bias": "v.b",
+             "q_norm": "q.norm", "k_norm": "k.norm"}
+
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        hidden, nq, nkv, d = (params[k] for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
+        dv = params.get("value_dim", d)
+        n = cls.tensor_names(params)
+        specs = {
+            n["q"]: TensorSpec((nq * d, hidden), fan_in=hidden),
+            n["k"]: TensorSpec((nkv * d, hidden), fan_in=hidden),
+            n["v"]: TensorSpec((nkv * dv, hidden), fan_in=hidden),
+            n["o"]: TensorSpec((hidden, nq * dv), fan_in=nq * dv),
+        }
+        if params.get("bias", False):
+            specs[n["q_bias"]] = TensorSpec((nq * d,), fan_in=hidden)
+            specs[n["k_bias"]] = TensorSpec((nkv * d,), fan_in=hidden)
+            specs[n["v_bias"]] = TensorSpec((nkv * dv,), fan_in=hidden)
+        if params.get("qk_norm", False):
+            specs[n["q_norm"]] = TensorSpec((nq * d,), kind="norm")
+            specs[n["k_norm"]] = TensorSpec((nkv * d,), kind="norm")
+        return specs
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries, weight_bytes: int, cache_bytes: int) -> StepCost:
+        """The projections; scores over head_dim channels and weighted values over value_dim channels for every key a
+        token sees; every request's visible keys and values read once, as wide as they are stored."""
+        cost = Part.step_cost.__func__(cls, params, entries, weight_bytes, cache_bytes)
+        nq, nkv, d, window = params["num_heads"], params["num_kv_heads"], params["head_dim"], params.get("window")
+        dv = params.get("value_dim", d)
+        for start, count in entries:
+            seen = 0
+            for p in range(start, start + count):
+                seen += min(p + 1, window) if window else p + 1
+            cost.flops += 2.0 * nq * (d + dv) * seen
+            context = start + count
+            kept = min(context, window + count - 1) if window else context
+            cost.cache_bytes += 2.0 * nkv * stored_width(d, dv) * cache_bytes * kept
+        return cost
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.hidden = int(params["hidden_size"])
+        self.nq = int(params["num_heads"])
+        self.nkv = int(params["num_kv_heads"])
+        self.qk_dim = int(params["head_dim"])
+        self.v_dim = int(params.get("value_dim", self.qk_dim))
+        if self.nq % self.nkv:
+            raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} key/value heads")
+        self.d = stored_width(self.qk_dim, self.v_dim)     # what the cache and the attention kernels see
+        self.scale = float(params["scale"])
+        self.window = params.get("window")
+        if self.window is not None and int(self.window) <= 0:
+            raise ValueError(f"an attention window must be positive, got {self.window}")
+        norm = params.get("qk_norm", False)
+        if norm not in (False, "projection"):
+            raise ValueError(f"attention_rows norms q and k over the 'projection' or not at all, got {norm!r}")
+        self.row_norm = norm == "projection"
+        self.eps = float(params.get("qk_norm_eps", 0.0))
+        self.out_scale = float(params.get("out_scale", 1.0))
+        self.position = params.get("position")
+        self.encodings = build.positions
+        if self.position is not None and self.position not in self.encodings:
+            raise KeyError(f"attention refers to position encoding '{self.position}', the model defines "
+                           f"{sorted(self.encodings)}")
+        load = build.loader
+        n = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
+        self.qkv = Linear(load.get_concat([n["q"], n["k"], n["v"]]), build.mode)
+        self.biases = tuple(load.get(n[k]) for k in ("q_bias", "k_bias", "v_bias")) if params.get("bias", False) else None
+        self.norm_weights = (load.get(n["q_norm"]), load.get(n["k_norm"])) if self.row_norm else None
+        o = load.get(n["o"])
+        if self.d != self.v_dim:   # zero columns where the stored heads hold zero value channels
+            wide = o.new_zeros(self.hidden, self.nq, self.d)
+            wide[:, :, :self.v_dim] = o.view(self.hidden, self.nq, self.v_dim)
+            o = wide.view(self.hidden, self.nq * self.d).contiguous()
+        self._o_weight = o
+        self._o = None
+        self.mode = build.mode
+        self.inner_width = self.nq * self.d
+        self.act_dtype = build.act_dtype
+        self.options = build.options
+        # what the inherited kernel choice asks about (none of it applies here)
+        self.qk_norm = self.plain_norm = self.values_are_keys = self.output_gate = False
+        self.q_temperature = None
+        self.q_w = self.k_w = None
+
+    accepts_residual = False
+    accepts_lazy_input = False
+    records_cleanly = True
+
+    def cache_spec(self) -> PagedKVSpec:
+        return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
+
+    def out_weight(self) -> torch.Tensor:
+        return self._o_weight
+
+    def forward_inner(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView, out: torch.Tensor) -> None:
+        tokens = x.shape[0]
+        ws = ctx.workspace
+        write = cache.writable
+        rows = None if write else self.nq * self.qk_dim
+        cols = self.qkv.out_features if rows is None else rows
+        qkv = ws.buffer("attention_rows.qkv", tokens, cols, self.act_dtype)
+        self.qkv.forward(x, qkv, rows=rows)
+        tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
+        table = ctx.block_tables[cache.group]
+        q = ws.buffer("attention_rows.q", tokens, self.nq * self.d, self.act_dtype)
+        kernels.qkv_rows(qkv, q, self.nq, self.nkv, self.qk_dim, self.v_dim, self.d, self.biases, self.norm_weights,
+                         self.eps, tables.cos if tables is not None else None,
+                         tables.sin if tables is not None else None, tables.rotary_dim if tables is not None else 0,
+                         tables.pairing if tables is not None else 0, cache.keys, cache.values, ctx.positions,
+                         ctx.token_entry, table, write_kv=write, value_scale=self.out_scale, norm=self.row_norm)
+        self.attend(q, out, ctx, cache, table)
+
+    def decodes_from_raw(self, ctx, cache, qkv, tables) -> bool:
+        return False
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView) -> torch.Tensor:
+        if self._o is None:
+            self._o = Linear(self._o_weight, self.mode)
+        ws = ctx.workspace
+        inner = ws.buffer("attention_rows.inner", x.shape[0], self.inner_width, self.act_dtype)
+        self.forward_inner(x, ctx, cache, inner)
+        return self._o.forward(inner, ws.buffer("attention_rows.out", x.shape[0], self.hidden, self.act_dtype))

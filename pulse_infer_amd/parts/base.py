@@ -232,11 +232,15 @@ class ResidualStream:
         self.stats: Optional[RowStats] = None
         self.after_block: Any = None   # the norm that reads the residual first once the block in hand is through
                                        # (set by whoever runs the blocks; None: unknown, or no norm)
+        self.copy: Optional[torch.Tensor] = None   # ``h`` once more in the activations' type, left by a block whose
+                                                   # sublayers read the stream itself; dropped when ``h`` changes
 
     def pending_for(self, norm: Any) -> Optional[torch.Tensor]:
         """The update not yet added, in a form ``norm`` takes: an update in parts ([parts, T, H] float32, the shares of
         a product whose inner dimension was split) is added to ``h`` first unless the norm says ``takes_parts``."""
         pending, self.pending = self.pending, None
+        if pending is not None:
+            self.copy = None
         if pending is not None and pending.dim() == 3 and not getattr(norm, "takes_parts", False):
             from ..ops import kernels
             kernels.residual_add(self.h, pending)
@@ -261,10 +265,12 @@ class ResidualStream:
             from ..ops import kernels
             kernels.residual_add(self.h, self.pending)
             self.pending = None
+            self.copy = None
 
     def push(self, delta: Any) -> None:
         """Hand over an update ([T, H], or [parts, T, H] float32 to be added in order); None or RowStats mean the part
         has already added it to ``h``."""
+        self.copy = None
         if isinstance(delta, RowStats):
             self.stats = delta
             return

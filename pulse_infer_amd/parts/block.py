@@ -7,13 +7,20 @@ the next norm's kernel through ``ResidualStream``.
 ``parallel``: n = norm(h); h <- h + (mixer(n) + ffn(n)): one norm, whose output both
 sublayers read; a layer may have no feed-forward (``LayerSpec.ffn`` None), then
 h <- h + mixer(norm(h)).
+
+``postnorm``: h <- norm_a(alpha h + ls_a * mixer(h)); h <- norm_b(alpha h + ls_b * ffn(h)): the
+sublayers read the stream itself, the norm comes after the sum, ``alpha`` weighs the
+stream in it and ``ls`` are optional factors, one a column, on a sublayer's result.
 """
 from __future__ import annotations
 
 from typing import Any, Dict, Optional
 
+import torch
+
 from ..models.spec import LayerSpec
 from ..weights.store import TensorSpec
+from ..ops import kernels
 from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, ResidualStream, StepContext, joined, says
 
 
@@ -171,3 +178,89 @@ class ParallelBlock(PreNormBlock):
             stream.push(self.ffn.forward(x, ctx, residual=stream.h, **self._told(stream.after_block)))
         else:
             stream.push(self.ffn.forward(x, ctx))
+
+
+@BLOCKS.register("postnorm")
+class PostNormBlock(Part):
+    """The norm after the sum.  Block parameters: ``alpha`` (the stream's weight in the sum, default 1);
+    ``mixer_norm`` / ``ffn_norm``: the norms' tensor prefixes below the layer's; ``mixer_scale`` / ``ffn_scale``: names
+    of the column factors on the sublayers' results (absent: none).  The norms are RMSNorms with plain weights
+    (``LayerSpec.norms`` gives their size and eps).  A layer without a feed-forward ends after the first norm.
+
+    The float32 stream is the normed rows themselves; a copy in the activations' type, which the sublayers'
+    products read, comes out of the same kernel (``ResidualStream.copy``).  A feed-forward may return two updates
+    (``returns_two``), which the kernel adds both."""
+
+    NORM_PLACES = ("mixer_norm", "ffn_norm")
+
+    @classmethod
+    def layer_weight_specs(cls, layer: LayerSpec) -> Dict[str, TensorSpec]:
+        p = layer.block.params
+        out: Dict[str, TensorSpec] = {}
+        places = [("mixer_norm", "mixer_scale")] + ([("ffn_norm", "ffn_scale")] if layer.ffn is not None else [])
+        for which, factors in places:
+            norm = layer.norm(which)
+            if norm.kind != "rmsnorm" or float(norm.params.get("weight_offset", 0.0)) != 0.0:
+                raise ValueError("the postnorm block takes RMSNorms with plain weights")
+            for name, spec in NORMS.get(norm.kind).weight_specs(norm.params).items():
+                out[joined(joined(layer.prefix, p[which]), name)] = spec
+            if p.get(factors):
+                out[joined(layer.prefix, p[factors])] = TensorSpec((norm.params["size"],), kind="norm")
+        parts = [(layer.mixer, MIXERS)] + ([(layer.ffn, FEED_FORWARDS)] if layer.ffn is not None else [])
+        for part, registry in parts:
+            sub = joined(layer.prefix, part.params.get("prefix", ""))
+            for name, spec in registry.get(part.kind).weight_specs(part.params).items():
+                out[joined(sub, name)] = spec
+        return out
+
+    def __init__(self, layer: LayerSpec, build: BuildContext):
+        p = layer.block.params
+        self.alpha = float(p.get("alpha", 1.0))
+        self.mixer = MIXERS.get(layer.mixer.kind)(layer.mixer.params,
+                                                  joined(layer.prefix, layer.mixer.params.get("prefix", "")), build)
+        self.ffn = None
+        if layer.ffn is not None:
+            self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
+                                                         joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
+        places = [("mixer_norm", "mixer_scale")] + ([("ffn_norm", "ffn_scale")] if self.ffn is not None else [])
+        self.norms = {}
+        for which, factors in places:
+            norm = layer.norm(which)
+            made = NORMS.get(norm.kind)(norm.params, joined(layer.prefix, p[which]), build)
+            scale = build.loader.get(joined(layer.prefix, p[factors])) if p.get(factors) else None
+            if scale is not None and scale.dtype != made.weight.dtype:
+                scale = scale.to(made.weight.dtype)
+            self.norms[which] = (made, scale)
+        self.act_dtype = build.act_dtype
+
+    def cache_spec(self) -> Optional[Any]:
+        return self.mixer.cache_spec()
+
+    def records_cleanly(self) -> bool:
+        return all(says(part, "records_cleanly") for part in (self.mixer, self.ffn) if part is not None)
+
+    def _rows(self, stream: ResidualStream, ctx: StepContext) -> torch.Tensor:
+        """The stream in the activations' type: itself in a float32 run, else the copy the last norm left (or one made
+        now, for the first block behind the embedding)."""
+        if self.act_dtype == torch.float32:
+            return stream.h
+        stream.settle()
+        if stream.copy is None:
+            stream.copy = ctx.workspace.buffer("block.rows", ctx.num_tokens, stream.h.shape[1], self.act_dtype)
+            kernels.round_rows(stream.h, stream.copy)
+        return stream.copy
+
+    def _close(self, stream: ResidualStream, ctx: StepContext, which: str, update: Any) -> None:
+        norm, scale = self.norms[which]
+        first, second = update if isinstance(update, tuple) else (update, None)
+        copy = None
+        if self.act_dtype != torch.float32:
+            copy = ctx.workspace.buffer("block.rows", ctx.num_tokens, stream.h.shape[1], self.act_dtype)
+        kernels.scale_add_rmsnorm(stream.h, norm.weight, norm.eps, self.alpha, first, second, scale, copy)
+        stream.stats = None
+        stream.copy = copy
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+        self._close(stream, ctx, "mixer_norm", self.mixer.forward(self._rows(stream, ctx), ctx, cache))
+        if self.ffn is not None:
+            self._close(stream, ctx, "ffn_norm", self.ffn.forward(self._rows(stream, ctx), ctx))

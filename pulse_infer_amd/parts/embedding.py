@@ -37,13 +37,14 @@ class TokenEmbedding(Part):
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
         self.table = build.loader.get(params["name"])
+        self.scale = float(params.get("scale", 1.0))   # every gathered row is multiplied by it, in float32
         self.bad_id = torch.zeros(1, dtype=torch.int32, device=build.device)
 
     def forward(self, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """The step function checks ids on the host before it runs.  A caller that comes another way and brings an
         id outside the table gets a row of NaN, which reaches that token's logits (no token is chosen from them),
         never a silent row of zeros; ``saw_bad_id`` tells, at the price of a synchronisation."""
-        kernels.embed_gather(ids, self.table, out, self.bad_id)
+        kernels.embed_gather(ids, self.table, out, self.bad_id, self.scale)
         return out
 
     def saw_bad_id(self, clear: bool = True) -> bool:
@@ -80,7 +81,14 @@ class OutputHead(Part):
         else:
             raise KeyError(f"'{params['name']}' is missing and the configuration does not tie it to the embedding")
         self.linear = Linear(weight, build.mode)
+        cap = params.get("softcap")
+        self.softcap = float(cap) if cap else 0.0   # logits <- cap * tanh(logits / cap)
+        if self.softcap < 0.0:
+            raise ValueError(f"a logit soft cap must be positive, got {self.softcap}")
 
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """out: float32 [R, vocab]."""
-        return self.linear.forward(x, out)
+        self.linear.forward(x, out)
+        if self.softcap:
+            kernels.softcap(out, self.softcap)
+        return out

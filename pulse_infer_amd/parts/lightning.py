@@ -1,0 +1,121 @@
+"""Linear attention with a constant decay per head ("lightning attention").
+
+For a token with input x: q = act(Wq x), k = act(Wk x) (heads x dim), v = act(Wv x) (heads x vdim), act = silu.
+Every head h keeps a state S [dim, vdim] per request, float32, zero at the request's start:
+
+    S <- decay_h S + k v^T          o = S^T q
+
+The heads' outputs of a token, taken together, are divided by their root mean square (eps), multiplied by a weight
+and by sigmoid(Wg x), and projected by Wo.  The four input projections are one product with the row-stacked weight;
+the recurrence is one kernel for prompts' portions and decoded tokens alike (``csrc/lightning.hip``); norm, gate and
+the one rounding are a second kernel.
+
+Parameters: ``hidden_size``, ``num_heads``, ``head_dim``, ``value_dim``, ``decay`` (one number a head), ``norm_eps``,
+``activation`` ("silu" or "none"), ``names`` (tensor names below the prefix), ``out_scale`` (a factor on the result).
+
+The part keeps a ``StateSpec`` per run.  It also answers the protocol of a branch of ``side_by_side``:
+``inner_width``, ``out_weight()`` and ``forward_inner(x, ctx, cache, out)``.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, List, Tuple
+
+import torch
+
+from ..cache.specs import StateSpec, StateView
+from ..ops import kernels
+from ..weights.store import TensorSpec
+from .base import MIXERS, BuildContext, Part, StepContext, StepCost, joined
+from .linear import Linear
+
+
+@MIXERS.register("lightning")
+class LightningAttention(Part):
+    NAMES = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o", "norm": "norm"}
+
+    @classmethod
+    def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
+        return {**cls.NAMES, **params.get("names", {})}
+
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        hidden, heads, d, dv = (params[k] for k in ("hidden_size", "num_heads", "head_dim", "value_dim"))
+        n = cls.tensor_names(params)
+        return {
+            n["q"]: TensorSpec((heads * d, hidden), fan_in=hidden),
+            n["k"]: TensorSpec((heads * d, hidden), fan_in=hidden),
+            n["v"]: TensorSpec((heads * dv, hidden), fan_in=hidden),
+            n["gate"]: TensorSpec((heads * dv, hidden), fan_in=hidden),
+            n["o"]: TensorSpec((hidden, heads * dv), fan_in=heads * dv),
+            n["norm"]: TensorSpec((heads * dv,), kind="norm"),
+        }
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries: List[Tuple[int, int]], weight_bytes: int,
+                  cache_bytes: int) -> StepCost:
+        """The projections, the recurrence (two multiply-adds a state element and token) and every request's state
+        read and written once, in float32."""
+        cost = super().step_cost(params, entries, weight_bytes, cache_bytes)
+        state = params["num_heads"] * params["head_dim"] * params["value_dim"]
+        rows = sum(count for _, count in entries)
+        cost.flops += 4.0 * state * rows
+        cost.cache_bytes += 8.0 * state * len(entries)
+        return cost
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.hidden = int(params["hidden_size"])
+        self.heads = int(params["num_heads"])
+        self.d = int(params["head_dim"])
+        self.dv = int(params["value_dim"])
+        decay = [float(v) for v in params["decay"]]
+        if len(decay) != self.heads:
+            raise ValueError(f"lightning attention of {self.heads} heads got {len(decay)} decays")
+        if self.d > 256:
+            raise ValueError(f"lightning attention takes at most 256 key channels a head, got {self.d}")
+        self.activation = params.get("activation", "silu")
+        if self.activation not in ("silu", "none"):
+            raise ValueError(f"lightning attention has no kernel for activation '{self.activation}'")
+        self.eps = float(params["norm_eps"])
+        self.out_scale = float(params.get("out_scale", 1.0))
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=build.device)
+        load = build.loader
+        self.names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
+        n = self.names
+        self.proj = Linear(load.get_concat([n["q"], n["k"], n["v"], n["gate"]]), build.mode)
+        self.norm_weight = load.get(n["norm"])
+        self._o_weight = load.get(n["o"])
+        self._o = None
+        self.mode = build.mode
+        self.act_dtype = build.act_dtype
+        self.inner_width = self.heads * self.dv
+
+    records_cleanly = True   # slots, starts and rows are read on the device
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.heads, self.d, self.dv), "float32")
+
+    def out_weight(self) -> torch.Tensor:
+        """Wo [hidden, inner_width]: what multiplies the rows ``forward_inner`` writes."""
+        return self._o_weight
+
+    def forward_inner(self, x: torch.Tensor, ctx: StepContext, cache: StateView, out: torch.Tensor) -> None:
+        """The mixer up to its output projection: ``out`` [T, inner_width] (rows may be strided) receives the normed,
+        gated heads times ``out_scale``."""
+        tokens = x.shape[0]
+        ws = ctx.workspace
+        hd, hv = self.heads * self.d, self.heads * self.dv
+        y = ws.buffer("lightning.proj", tokens, 2 * hd + 2 * hv, self.act_dtype)
+        self.proj.forward(x, y)
+        o = ws.buffer("lightning.heads", tokens, hv, torch.float32)
+        groups = kernels.lightning_row_groups(len(ctx.entries), self.heads, self.d, self.dv)
+        kernels.lightning_scan(y, 0, hd, 2 * hd, o, cache.state, self.decay, ctx.entry_first_row, ctx.entry_start,
+                               ctx.entry_slot, self.heads, self.d, self.dv, self.activation, groups)
+        kernels.gated_rmsnorm(o, self.norm_weight, y[:, 2 * hd + hv:], out, self.eps, self.out_scale)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: StateView) -> torch.Tensor:
+        if self._o is None:
+            self._o = Linear(self._o_weight, self.mode)
+        ws = ctx.workspace
+        inner = ws.buffer("lightning.inner", x.shape[0], self.inner_width, self.act_dtype)
+        self.forward_inner(x, ctx, cache, inner)
+        return self._o.forward(inner, ws.buffer("lightning.out", x.shape[0], self.hidden, self.act_dtype))

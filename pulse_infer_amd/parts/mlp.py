@@ -90,3 +90,43 @@ class GatedMLP(Part):
         if residual is not None:
             return self.down.add_into(z, residual, out, ws, next_scale, next_offset, leave_stats)
         return self.down.forward(z, out)
+
+
+@FEED_FORWARDS.register("mlp")
+class PlainMLP(Part):
+    """down(act(up(x))), no gate and no biases.  Parameters: ``hidden_size``, ``intermediate_size``, ``activation``
+    ("relu2": the square of relu, "gelu_tanh", "silu"), ``names`` (``up``, ``down``)."""
+
+    NAMES = {"up": "up", "down": "down"}
+
+    @classmethod
+    def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
+        return {**cls.NAMES, **params.get("names", {})}
+
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        hidden, inter = params["hidden_size"], params["intermediate_size"]
+        names = cls.tensor_names(params)
+        return {names["up"]: TensorSpec((inter, hidden), fan_in=hidden),
+                names["down"]: TensorSpec((hidden, inter), fan_in=inter)}
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.hidden = int(params["hidden_size"])
+        self.inter = int(params["intermediate_size"])
+        self.activation = params.get("activation", "relu2")
+        if self.activation not in kernels.ACTIVATIONS:
+            raise ValueError(f"mlp has no kernel for activation '{self.activation}' (known: {sorted(kernels.ACTIVATIONS)})")
+        names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
+        self.up = Linear(build.loader.get(names["up"]), build.mode)
+        self.down = Linear(build.loader.get(names["down"]), build.mode)
+        self.act_dtype = build.act_dtype
+
+    records_cleanly = True
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        tokens = x.shape[0]
+        ws = ctx.workspace
+        z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
+        self.up.forward(x, z)
+        kernels.activation(z, z, self.activation)
+        return self.down.forward(z, ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype))

@@ -1,0 +1,123 @@
+"""A routed feed-forward: every token goes through the few experts its router chooses.
+
+Router: z = Wr x in float32; s = softmax(z) over all router outputs; the ``top`` outputs with the largest
+s + correction are chosen; their weights are their s divided by the sum of the chosen s (+ 1e-20).  The first
+``num_experts`` outputs are gated feed-forwards, down_e(silu(gate_e x) * (up_e x)), without biases; the last
+``num_identity`` outputs are identity experts, whose result is x itself and which have no tensors.  The result is the
+weighted sum over the chosen outputs; a shared expert of the same form (``shared_size``, optional) runs for every
+token and is added.
+
+Parameters: ``hidden_size``, ``expert_size``, ``num_experts``, ``num_identity``, ``top``, ``correction`` (whether a
+correction tensor exists), ``shared_size`` (None: no shared expert), ``names``: ``router``, ``correction``,
+``expert`` (a pattern with ``{e}``), ``gate`` / ``up`` / ``down`` (below an expert's or the shared expert's prefix),
+``shared``.
+
+The experts' weights are stacked at load time ([experts, rows, columns]).  ``forward`` returns the routed part
+(float32) and the shared expert's part as two updates that the block adds.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, List, Optional, Tuple
+
+import torch
+
+from ..ops import kernels
+from ..weights.store import TensorSpec
+from .base import FEED_FORWARDS, BuildContext, Part, StepContext, StepCost, joined
+from .mlp import GatedMLP
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(Part):
+    NAMES = {"router": "router", "correction": "correction", "expert": "e{e}", "gate": "gate", "up": "up",
+             "down": "down", "shared": "shared"}
+
+    @classmethod
+    def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
+        return {**cls.NAMES, **params.get("names", {})}
+
+    @classmethod
+    def _shared_params(cls, params: Dict[str, Any]) -> Optional[Dict[str, Any]]:
+        if params.get("shared_size") is None:
+            return None
+        n = cls.tensor_names(params)
+        return {"hidden_size": params["hidden_size"], "intermediate_size": params["shared_size"], "activation": "silu",
+                "names": {"gate": n["gate"], "up": n["up"], "down": n["down"]}}
+
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        hidden, ff, experts = params["hidden_size"], params["expert_size"], params["num_experts"]
+        outputs = experts + params.get("num_identity", 0)
+        n = cls.tensor_names(params)
+        specs = {n["router"]: TensorSpec((outputs, hidden), fan_in=hidden)}
+        if params.get("correction", False):
+            specs[n["correction"]] = TensorSpec((outputs,), kind="linear", fan_in=100 * outputs)
+        for e in range(experts):
+            sub = n["expert"].format(e=e)
+            specs[joined(sub, n["gate"])] = TensorSpec((ff, hidden), fan_in=hidden)
+            specs[joined(sub, n["up"])] = TensorSpec((ff, hidden), fan_in=hidden)
+            specs[joined(sub, n["down"])] = TensorSpec((hidden, ff), fan_in=ff)
+        shared = cls._shared_params(params)
+        if shared is not None:
+            for name, spec in GatedMLP.weight_specs(shared).items():
+                specs[joined(n["shared"], name)] = spec
+        return specs
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries: List[Tuple[int, int]], weight_bytes: int,
+                  cache_bytes: int) -> StepCost:
+        """Router and shared expert for every row; of the routed experts what the rows choose: ``top`` experts a row
+        in arithmetic (less the identity experts' share), and at most all experts' weights once."""
+        hidden, ff, experts = params["hidden_size"], params["expert_size"], params["num_experts"]
+        outputs = experts + params.get("num_identity", 0)
+        rows = sum(count for _, count in entries)
+        real = params["top"] * experts / float(outputs)
+        cost = StepCost(flops=2.0 * rows * outputs * hidden + 6.0 * rows * real * hidden * ff,
+                        weight_bytes=float(outputs * hidden * weight_bytes)
+                        + 3.0 * hidden * ff * weight_bytes * min(experts, rows * real))
+        shared = cls._shared_params(params)
+        if shared is not None:
+            cost = cost + GatedMLP.step_cost(shared, entries, weight_bytes, cache_bytes)
+        return cost
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.hidden = int(params["hidden_size"])
+        self.ff = int(params["expert_size"])
+        self.experts = int(params["num_experts"])
+        self.identity = int(params.get("num_identity", 0))
+        self.top = int(params["top"])
+        outputs = self.experts + self.identity
+        if not 0 < self.top <= outputs:
+            raise ValueError(f"a router with {outputs} outputs cannot choose {self.top}")
+        if self.experts <= 0:
+            raise ValueError("routed_experts needs at least one expert with weights")
+        load = build.loader
+        n = self.tensor_names(params)
+        self.router = load.get(joined(prefix, n["router"]))
+        self.correction = load.get(joined(prefix, n["correction"])) if params.get("correction", False) else None
+        stack = lambda which: torch.stack([load.get(joined(joined(prefix, n["expert"].format(e=e)), n[which]))
+                                           for e in range(self.experts)], dim=0).contiguous()
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        shared = self._shared_params(params)
+        self.shared = GatedMLP(shared, joined(prefix, n["shared"]), build) if shared is not None else None
+        self.act_dtype = build.act_dtype
+        self.device = build.device
+
+    records_cleanly = True   # choices stay on the device; the launches do not depend on them
+    returns_two = True       # forward gives (routed update, shared update or None)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext):
+        tokens = x.shape[0]
+        ws = ctx.workspace
+        outputs = self.experts + self.identity
+        z = ws.buffer("moe.logits", tokens, outputs, torch.float32)
+        kernels.gemm_f32(x, self.router, z)
+        idx = ws.buffer("moe.idx", tokens, self.top, torch.int32)
+        weight = ws.buffer("moe.weight", tokens, self.top, torch.float32)
+        kernels.moe_route(z, self.correction, self.top, idx, weight)
+        act = ws.buffer("moe.act", tokens * self.top, self.ff, self.act_dtype)
+        kernels.moe_gate_up(x, self.w_gate, self.w_up, idx, act)
+        routed = ws.buffer("moe.out", tokens, self.hidden, torch.float32)
+        kernels.moe_down(x, act, self.w_down, idx, weight, routed)
+        shared = self.shared.forward(x, ctx) if self.shared is not None else None
+        return routed, shared
