@@ -125,7 +125,7 @@ def check(name, args):
         gu, out, _, tokens, inter, _, _ = args
         need(room(gu) >= val(tokens) * 2 * val(inter) and room(out) >= val(tokens) * val(inter), "operands")
     elif name == "pulse_embed_gather":
-        ids, _, _, out, tokens, hidden, _, _, _ = args
+        ids, _, _, out, tokens, hidden, _, _, _, _ = args
         need(room(out) >= val(tokens) * val(hidden) and room(ids) >= val(tokens), "operands")
     elif name == "pulse_residual_add":
         h, delta, _, parts, n, _ = args
