@@ -55,13 +55,13 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     p.add_argument("--model", choices=sorted(SHAPES), default="8b", help="layer sizes: Qwen3-8B (the default), 14B or 32B")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has, if memory or time needs it")
-    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen"], default="decode",
+    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen", "kesovik"], default="decode",
                    help="decode: fixed batch at a fixed context; serving: continuous batching of requests with "
                         "seeded prompt lengths, chunked prefill mixed with decoding; long-prompt: one prompt of "
-                        "--prompt-tokens tokens in portions of --chunk tokens; dirozen: decoding and prefill of the "
-                        "Dirozen design beside Qwen3 layers of equal sizes, with both models' time by entry point")
-    p.add_argument("--compare-layers", type=int, default=4, help="dirozen: layers of the two models that are compared")
-    p.add_argument("--compare-sizes", default="2k,4k,5k", help="dirozen: which of the layer sizes 2k, 4k, 5k (widths) to run")
+                        "--prompt-tokens tokens in portions of --chunk tokens; dirozen / kesovik: decoding and prefill of "
+                        "that design beside Qwen3 layers of equal sizes, with both models' time by entry point")
+    p.add_argument("--compare-layers", type=int, default=4, help="dirozen, kesovik: layers of the two models that are compared")
+    p.add_argument("--compare-sizes", default="2k,4k,5k", help="dirozen, kesovik: which of the layer sizes 2k, 4k, 5k (widths) to run")
     p.add_argument("--prompt-tokens", type=int, default=16384, help="long-prompt: length of the prompt")
     p.add_argument("--requests", type=int, default=32, help="serving: number of requests")
     p.add_argument("--prompt-range", type=int, nargs=2, default=[128, 2048], help="serving: prompt lengths drawn from [lo, hi]")
@@ -231,15 +231,36 @@ DIROZEN_SIZES = {   # layer sizes of the comparison: width, query heads, key/val
 }
 
 
-def dirozen_compare(args) -> int:
-    """Dirozen beside Qwen3 layers of equal sizes (random weights, ``--compare-layers`` layers, a vocabulary of
+def kesovik_layers(size, layers):
+    """Kesovik layers at the comparison's sizes, in turn: two mixers side by side (window attention over 1,024 tokens
+    beside lightning attention with half as many heads) with a dense feed-forward, the same with routed experts,
+    lightning attention alone with routed experts, the first again.  The routed feed-forward has 16 experts and 2
+    identity experts, 4 chosen a token, each an eighth as wide as the dense one, and a shared expert a quarter as
+    wide: three quarters of the dense feed-forward's arithmetic a token."""
+    left = {"dim": size["dim"], "heads": size["heads"], "kv_heads": size["kv_heads"], "mask": {"size": 1024},
+            "rot": {"base": 1e6, "dims": size["dim"]}, "scale": size["dim"] ** -0.5, "vdim": size["dim"]}
+    def lightning(heads):
+        decay = [1.0 - 2.0 ** -(5 + 8.0 * h / heads) for h in range(heads)]
+        return {"decay": decay, "dim": size["dim"], "heads": heads, "vdim": size["dim"]}
+    both = {"left": left, "left_scale": 0.8, "right": lightning(size["heads"] // 2), "right_scale": 1.1}
+    dense = {"ff": size["ff"], "kind": "dense"}
+    routed = {"expert": {"ff": size["ff"] // 8}, "kind": "moe", "router": {"experts": 16, "identity": 2, "top": 4},
+              "shared": {"ff": size["ff"] // 4}}
+    turn = [{"type": "parallel", "mixer": both, "mlp": dense}, {"type": "parallel", "mixer": both, "mlp": routed},
+            {"type": "lightning", "mixer": lightning(size["heads"]), "mlp": routed},
+            {"type": "parallel", "mixer": both, "mlp": dense}]
+    return [turn[i % len(turn)] for i in range(layers)]
+
+
+def dirozen_compare(args, design: str = "dirozen") -> int:
+    """Dirozen (or, with ``design`` "kesovik", Kesovik) beside Qwen3 layers of equal sizes (random weights, ``--compare-layers`` layers, a vocabulary of
     32,000): decoding at batch 1 / 8 / 32 with contexts ending at ``--context`` and a prompt of ``--prefill-tokens``
     tokens, each through the engine's own serving loop, with the fraction of the roofline from the models' own
     descriptions, and where an eager decoding step and a prompt step spend their time by entry point.  One JSON
     line."""
     import torch
 
-    from pulse_infer_amd.config import DirozenConfig, Qwen3Config
+    from pulse_infer_amd.config import DirozenConfig, KesovikConfig, Qwen3Config
     from pulse_infer_amd.engine.engine import ContinuousBatchEngine
     from pulse_infer_amd.engine.runner import StepEntry
     from pulse_infer_amd.models.causal_lm import expected_tensors
@@ -269,6 +290,12 @@ def dirozen_compare(args) -> int:
                  "mlp": {"ff": size["ff"], "kind": "dense"}}
         dirozen = DirozenConfig.from_dict({"architecture": "Dirozen", "vocab": vocab, "width": size["width"],
                                            "norm": {"eps": 1e-6}, "layers": [entry] * layers}, "<bench>")
+        if design == "kesovik":
+            kesovik = KesovikConfig.from_dict({
+                "architecture": "Kesovik", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-6},
+                "embedding": {"scale": 1.0}, "postln_alpha": 2.0, "logit_softcap": 30.0,
+                "layers": kesovik_layers(size, layers)}, "<bench>")
+            return {"kesovik": kesovik, "qwen3": qwen}
         return {"dirozen": dirozen, "qwen3": qwen}
 
     def measure(cfg):
@@ -283,6 +310,8 @@ def dirozen_compare(args) -> int:
         for g in runner.cache.groups:
             for t in g.spec.tensors(g.storage):
                 t.normal_(0.0, 1.0)
+        for state in runner.cache.state.values():     # requests admitted as computed continue from what lies there
+            state.normal_(0.0, 0.1)
         gen = torch.Generator().manual_seed(args.seed)
         out = {}
         steps, warmup = max(8, min(args.steps, 32)), max(4, min(args.warmup, 8))
@@ -350,21 +379,23 @@ def dirozen_compare(args) -> int:
         torch.cuda.empty_cache()
         return out
 
-    record = {"metric": "dirozen_beside_qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
+    record = {"metric": f"{design}_beside_qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
               "data": "synthetic", "layers": layers, "vocab": vocab, "context": args.context, "sizes": {}}
     for name, size in DIROZEN_SIZES.items():
         if name not in args.compare_sizes.split(","):
             continue
         both = {model: measure(cfg) for model, cfg in configs(size).items()}
-        ratio = {k: round(both["dirozen"][k]["tokens_per_s"] / both["qwen3"][k]["tokens_per_s"], 3)
-                 for k in both["dirozen"] if "tokens_per_s" in both["dirozen"][k]}
-        record["sizes"][name] = dict(size, **both, dirozen_over_qwen3=ratio)
+        ratio = {k: round(both[design][k]["tokens_per_s"] / both["qwen3"][k]["tokens_per_s"], 3)
+                 for k in both[design] if "tokens_per_s" in both[design][k]}
+        record["sizes"][name] = dict(size, **both, **{f"{design}_over_qwen3": ratio})
     print(json.dumps(record))
     return 0
 
 
 def main() -> int:
     args = parse_args()
+    if args.workload == "kesovik":
+        return dirozen_compare(args, "kesovik")
     if args.workload == "dirozen":
         if args.gpus != 1:
             print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

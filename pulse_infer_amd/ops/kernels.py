@@ -817,3 +817,58 @@ def moe_down(x: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, idx: torc
           f"moe_down: out must be float32 [{tokens}, {hidden}]")
     call("pulse_moe_down", _ptr(x), _ptr(act), _i32(_tag(x, "moe_down")), _ptr(w_down), _i32(_tag(w_down, "moe_down")),
          _ptr(idx), _ptr(weight), _ptr(out), _i32(tokens), _i32(hidden), _i32(ff), _i32(experts), _i32(top), _stream())
+
+
+MOE_TILE_ROWS = (32, 128)   # rows of an expert's tile in the grouped products
+
+
+def moe_grouped_takes(x: torch.Tensor, w_gate: torch.Tensor, w_down: torch.Tensor) -> bool:
+    """Whether the experts' products run grouped on the matrix cores: bfloat16 everywhere, rows of multiples of 8."""
+    experts, ff, hidden = w_gate.shape
+    return (x.dtype == torch.bfloat16 and w_gate.dtype == torch.bfloat16 and w_down.dtype == torch.bfloat16
+            and hidden % 8 == 0 and ff % 8 == 0 and experts <= 1024 and x.data_ptr() % 16 == 0)
+
+
+def moe_max_tiles(pairs: int, experts: int, tile_rows: int) -> int:
+    """The most tiles a step of ``pairs`` (token, choice) pairs can have, however they choose."""
+    return (pairs + tile_rows - 1) // tile_rows + experts
+
+
+def moe_grouped(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor,
+                weight: torch.Tensor, act: torch.Tensor, y: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor,
+                tile_rows: int) -> None:
+    """out[t] = sum_k weight[t, k] * (expert idx[t, k] of x[t], or x[t] itself for an identity expert), the experts'
+    products grouped by expert on the matrix cores.  ``act`` bfloat16 [T * top, ff] and ``y`` float32 [T * top, hidden]
+    are scratch; ``scratch`` int32 holds 2 * T * top + 3 * moe_max_tiles + 1 entries."""
+    _gpu("moe_grouped", x, w_gate, w_up, w_down, idx, weight, act, y, out, scratch)
+    tokens, hidden = x.shape
+    experts, ff, h2 = w_gate.shape
+    top = idx.shape[1]
+    pairs = tokens * top
+    _need(moe_grouped_takes(x, w_gate, w_down) and w_up.dtype == torch.bfloat16, "moe_grouped: bfloat16 operands with rows of multiples of 8")
+    _need(tile_rows in MOE_TILE_ROWS, f"moe_grouped: tiles of {MOE_TILE_ROWS} rows")
+    _need(h2 == hidden and w_up.shape == w_gate.shape and tuple(w_down.shape) == (experts, hidden, ff)
+          and w_gate.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous() and x.is_contiguous(),
+          "moe_grouped: stacked contiguous weights [experts, ff, hidden] and [experts, hidden, ff]")
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and tuple(idx.shape) == (tokens, top)
+          and weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == (tokens, top),
+          "moe_grouped: idx int32 and weight float32 must be [T, top]")
+    _need(act.dtype == torch.bfloat16 and act.is_contiguous() and tuple(act.shape) == (pairs, ff)
+          and y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (pairs, hidden)
+          and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (tokens, hidden),
+          "moe_grouped: act, y or out of the wrong shape or storage type")
+    tiles = moe_max_tiles(pairs, experts, tile_rows)
+    _need(scratch.dtype == torch.int32 and scratch.is_contiguous() and scratch.numel() >= 2 * pairs + 3 * tiles + 1,
+          "moe_grouped: the integer scratch is too small")
+    base = scratch.data_ptr()
+    at = lambda n: ctypes.c_void_p(base + 4 * n)
+    rank, order = at(0), at(pairs)
+    t_expert, t_row0, t_rows, count = at(2 * pairs), at(2 * pairs + tiles), at(2 * pairs + 2 * tiles), at(2 * pairs + 3 * tiles)
+    call("pulse_moe_group", _ptr(idx), _i32(pairs), _i32(experts), _i32(tile_rows), _i32(tiles), rank, order, t_expert,
+         t_row0, t_rows, count, _stream())
+    call("pulse_moe_gate_up_grouped", _ptr(x), _ptr(w_gate), _ptr(w_up), order, t_expert, t_row0, t_rows, count, _i32(tiles),
+         _i32(tile_rows), _ptr(act), _i32(hidden), _i32(ff), _i32(top), _stream())
+    call("pulse_moe_down_grouped", _ptr(act), _ptr(w_down), order, t_expert, t_row0, t_rows, count, _i32(tiles),
+         _i32(tile_rows), _ptr(y), _i32(hidden), _i32(ff), _stream())
+    call("pulse_moe_combine", _ptr(x), _i32(_tag(x, "moe_grouped")), _ptr(y), _ptr(idx), _ptr(weight), _ptr(out),
+         _i32(tokens), _i32(hidden), _i32(experts), _i32(top), _stream())

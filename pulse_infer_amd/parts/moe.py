@@ -116,8 +116,17 @@ class RoutedExperts(Part):
         weight = ws.buffer("moe.weight", tokens, self.top, torch.float32)
         kernels.moe_route(z, self.correction, self.top, idx, weight)
         act = ws.buffer("moe.act", tokens * self.top, self.ff, self.act_dtype)
-        kernels.moe_gate_up(x, self.w_gate, self.w_up, idx, act)
         routed = ws.buffer("moe.out", tokens, self.hidden, torch.float32)
-        kernels.moe_down(x, act, self.w_down, idx, weight, routed)
+        if kernels.moe_grouped_takes(x, self.w_gate, self.w_down):
+            # bfloat16: the pairs grouped by expert on the device, every expert's rows on the matrix cores; tiles of
+            # 128 rows once an expert gets about that many
+            pairs = tokens * self.top
+            rows = kernels.MOE_TILE_ROWS[1] if pairs >= 64 * self.experts else kernels.MOE_TILE_ROWS[0]
+            y = ws.buffer("moe.y", pairs, self.hidden, torch.float32)
+            ints = ws.buffer("moe.ints", 2 * pairs + 3 * kernels.moe_max_tiles(pairs, self.experts, rows) + 1, 1, torch.int32)
+            kernels.moe_grouped(x, self.w_gate, self.w_up, self.w_down, idx, weight, act, y, routed, ints.view(-1), rows)
+        else:
+            kernels.moe_gate_up(x, self.w_gate, self.w_up, idx, act)
+            kernels.moe_down(x, act, self.w_down, idx, weight, routed)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         return routed, shared

