@@ -21,11 +21,10 @@ namespace {
 
 constexpr int ROUTE_PER_LANE = 16;   // router outputs <= 64 * 16
 
+// One wavefront routes one token: `row` holds its n router logits (in global memory or in LDS).
 template <typename TW>
-__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const TW* __restrict__ correction,
-                                                       int* __restrict__ idx, float* __restrict__ weight, int n, int top) {
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const float* row = z + static_cast<int64_t>(t) * n;
+__device__ __forceinline__ void route_row(const float* row, const TW* __restrict__ correction, int* __restrict__ idx,
+                                          float* __restrict__ weight, int n, int top, int t, int lane) {
     float s[ROUTE_PER_LANE], c[ROUTE_PER_LANE];
     float m = -INFINITY;
 #pragma unroll
@@ -81,6 +80,50 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
         idx[static_cast<int64_t>(t) * top + lane] = mine_idx;
         weight[static_cast<int64_t>(t) * top + lane] = mine / (total + 1e-20f);
     }
+}
+
+template <typename TW>
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const TW* __restrict__ correction,
+                                                       int* __restrict__ idx, float* __restrict__ weight, int n, int top) {
+    route_row<TW>(z + static_cast<int64_t>(blockIdx.x) * n, correction, idx, weight, n, top, blockIdx.x, threadIdx.x);
+}
+
+// The router's product and the routing in one: a workgroup a token holds the token's row in LDS, its wavefronts
+// take the router's outputs in turn (float32 multiply-adds over the hidden size, lanes sharing a dot product out),
+// and the first wavefront routes.
+template <typename TX, typename TW>
+__global__ __launch_bounds__(256) void moe_router_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
+                                                         const TW* __restrict__ correction, int* __restrict__ idx,
+                                                         float* __restrict__ weight, int hidden, int n, int top) {
+    extern __shared__ float x_s[];          // [hidden] then [n]
+    float* z_s = x_s + hidden;
+    const int t = blockIdx.x;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) x_s[i] = to_f32<TX>(x[static_cast<int64_t>(t) * hidden + i]);
+    __syncthreads();
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+    const bool wide = sizeof(TW) == 2 && hidden % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+    for (int o = wave; o < n; o += 4) {
+        const TW* wrow = w + static_cast<int64_t>(o) * hidden;
+        float sum = 0.f;
+        if (wide) {   // 16 bytes of a bfloat16 row a lane and step
+            for (int i = lane * 8; i < hidden; i += PULSE_WAVE * 8) {
+                const pulse_i32x4 raw = *reinterpret_cast<const pulse_i32x4*>(wrow + i);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t two = static_cast<uint32_t>(raw[u]);
+                    sum = fmaf(__uint_as_float(two << 16), x_s[i + 2 * u], sum);
+                    sum = fmaf(__uint_as_float(two & 0xffff0000u), x_s[i + 2 * u + 1], sum);
+                }
+            }
+        } else {
+#pragma unroll 4
+            for (int i = lane; i < hidden; i += PULSE_WAVE) sum = fmaf(to_f32<TW>(wrow[i]), x_s[i], sum);
+        }
+        sum = wave_sum(sum);
+        if (lane == 0) z_s[o] = sum;
+    }
+    __syncthreads();
+    if (wave == 0) route_row<TW>(z_s, correction, idx, weight, n, top, t, lane);
 }
 
 template <typename TX, typename TW>
@@ -158,6 +201,23 @@ extern "C" int pulse_moe_route(const float* z, const void* correction, int c_dty
     PULSE_DISPATCH_DTYPE(c_dtype, TW, hipLaunchKernelGGL(moe_route_kernel<TW>, dim3(tokens), dim3(64), 0, stream, z,
                                                          static_cast<const TW*>(correction), idx, weight, n, top));
     PULSE_LAUNCH_CHECK("moe_route");
+    return 0;
+}
+
+extern "C" int pulse_moe_router(const void* x, int x_dtype, const void* w, const void* correction, int w_dtype, int* idx,
+                                float* weight, int tokens, int hidden, int n, int top, hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && n > 0 && top > 0 && top <= n && x && w && idx && weight,
+                  "moe_router: bad arguments");
+    PULSE_REQUIRE(n <= PULSE_WAVE * ROUTE_PER_LANE && top <= PULSE_WAVE,
+                  "moe_router: at most %d router outputs and %d choices", PULSE_WAVE * ROUTE_PER_LANE, PULSE_WAVE);
+    PULSE_REQUIRE(pulse_dtype_ok(x_dtype) && pulse_dtype_ok(w_dtype), "moe_router: bad dtype tag");
+    const size_t lds = sizeof(float) * (static_cast<size_t>(hidden) + n);
+    PULSE_REQUIRE(lds <= 60 * 1024, "moe_router: rows of %d values do not fit the workgroup's memory", hidden);
+    if (tokens == 0) return 0;
+    PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
+        hipLaunchKernelGGL((moe_router_kernel<TX, TW>), dim3(tokens), dim3(256), lds, stream, static_cast<const TX*>(x),
+                           static_cast<const TW*>(w), static_cast<const TW*>(correction), idx, weight, hidden, n, top)));
+    PULSE_LAUNCH_CHECK("moe_router");
     return 0;
 }
 

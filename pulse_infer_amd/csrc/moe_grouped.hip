@@ -97,6 +97,53 @@ __device__ __forceinline__ void walk(const bf16_t* const (&wrow)[NW], const bf16
     }
 }
 
+// The same walk for tiles of 128 rows (RB = 8): the tile's rows go through LDS in pieces of 64 values of k, fetched
+// once by the workgroup's 256 threads (a thread half a row's piece: 64 bytes) instead of once by every wavefront, the
+// next piece travelling while this one is multiplied.  src[t]: the row that thread t fetches half of (null: none).
+constexpr int STAGE_K = 64;
+constexpr int STAGE_ROW = STAGE_K + 8;   // values a row takes in LDS (the 8 more keep rows off each other's banks)
+
+template <int NW>
+__device__ __forceinline__ void walk_staged(const bf16_t* const (&wrow)[NW], const bf16_t* src, bf16_t* stage, int blocks,
+                                            int K, int r, int kg, f32x4 (&acc)[NW][8]) {
+    const int tid = threadIdx.x;
+    const int frow = tid / 2, fk = (tid % 2) * 32;   // this thread fetches values fk .. fk + 31 of row frow's piece
+    bf16x8 held[4];
+    auto fetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int kc = k0 + fk + 8 * u;
+            held[u] = (src && kc < K) ? *reinterpret_cast<const bf16x8*>(src + kc) : zeros8();
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += STAGE_K) {
+        __syncthreads();   // the piece in LDS has been multiplied
+#pragma unroll
+        for (int u = 0; u < 4; ++u) *reinterpret_cast<bf16x8*>(stage + frow * STAGE_ROW + fk + 8 * u) = held[u];
+        __syncthreads();
+        if (k0 + STAGE_K < K) fetch(k0 + STAGE_K);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int kc = k0 + 32 * half + kg * 8;
+            const bool kok = kc < K;
+            bf16x8 wa[NW];
+#pragma unroll
+            for (int s = 0; s < NW; ++s)
+                wa[s] = (kok && wrow[s]) ? *reinterpret_cast<const bf16x8*>(wrow[s] + kc) : zeros8();
+#pragma unroll
+            for (int rb = 0; rb < 8; ++rb) {
+                if (rb < blocks) {
+                    const bf16x8 xb = *reinterpret_cast<const bf16x8*>(stage + (rb * 16 + r) * STAGE_ROW + 32 * half + kg * 8);
+#pragma unroll
+                    for (int s = 0; s < NW; ++s)
+                        acc[s][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[s], xb, acc[s][rb], 0, 0, 0);
+                }
+            }
+        }
+    }
+}
+
 template <int RB>
 __global__ __launch_bounds__(256) void moe_gate_up_grouped_kernel(const bf16_t* __restrict__ x,
                                                                   const bf16_t* __restrict__ wg,
@@ -129,7 +176,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_grouped_kernel(const bf16_t* 
     for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) acc[s][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-    walk<RB, 2>(wrow, xrow, (rows + 15) / 16, hidden, kg, acc);
+    if constexpr (RB == 8) {
+        __shared__ __attribute__((aligned(16))) bf16_t stage[128 * STAGE_ROW];
+        const int mine = threadIdx.x / 2;
+        const int p = mine < rows ? order[row0 + mine] : -1;
+        walk_staged<2>(wrow, p >= 0 ? x + static_cast<int64_t>(p / top) * hidden : nullptr, stage, (rows + 15) / 16, hidden,
+                       r, kg, acc);
+    } else {
+        walk<RB, 2>(wrow, xrow, (rows + 15) / 16, hidden, kg, acc);
+    }
     // lane l holds inner columns 4 * (l / 16) + i of this wavefront's 16, for row l % 16 of every block
     const int j0 = blockIdx.y * 64 + wave * 16 + 4 * kg;
 #pragma unroll
@@ -174,7 +229,14 @@ __global__ __launch_bounds__(256) void moe_down_grouped_kernel(const bf16_t* __r
     f32x4 acc[1][RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) acc[0][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-    walk<RB, 1>(wrow, xrow, (rows + 15) / 16, ff, kg, acc);
+    if constexpr (RB == 8) {
+        __shared__ __attribute__((aligned(16))) bf16_t stage[128 * STAGE_ROW];
+        const int mine = threadIdx.x / 2;
+        const int p = mine < rows ? order[row0 + mine] : -1;
+        walk_staged<1>(wrow, p >= 0 ? act + static_cast<int64_t>(p) * ff : nullptr, stage, (rows + 15) / 16, ff, r, kg, acc);
+    } else {
+        walk<RB, 1>(wrow, xrow, (rows + 15) / 16, ff, kg, acc);
+    }
     const int c0 = blockIdx.y * 64 + wave * 16 + 4 * kg;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {

@@ -75,7 +75,7 @@ extern "C" int pulse_scale_add_rmsnorm(float* h, const void* d1, int d1_dtype, c
     const size_t lds = sizeof(float) * static_cast<size_t>(hidden);
     PULSE_REQUIRE(lds <= 60 * 1024, "scale_add_rmsnorm: rows of %d values do not fit the workgroup's memory", hidden);
     if (rows == 0) return 0;
-    const int threads = hidden >= 2048 ? 1024 : 256;
+    const int threads = hidden >= 2048 || (rows <= 64 && hidden >= 1024) ? 1024 : 256;
     PULSE_DISPATCH_DTYPE(d1_dtype, T1, PULSE_DISPATCH_DTYPE(d2_dtype, T2, PULSE_DISPATCH_DTYPE(w_dtype, TW,
         PULSE_DISPATCH_DTYPE(copy_dtype, TY,
             hipLaunchKernelGGL((scale_add_rmsnorm_kernel<T1, T2, TW, TY>), dim3(rows), dim3(threads), lds, stream, h,

@@ -13,7 +13,8 @@
 // with zeros up to D channels (D >= d, dv): the attention kernels then see heads of one
 // width D, the zero channels add nothing to a score, and the value channels beyond dv
 // come out as zeros.  Everything is float32 until the one rounding of the store.
-// One workgroup a token.
+// One workgroup a token, or several that each redo the token's sums of squares and share its channels out (few
+// tokens: a decoding step).
 #include "common.h"
 
 #include <math.h>
@@ -90,7 +91,8 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
         return u;
     };
     TX* qrow = q_out + static_cast<int64_t>(t) * a.q_stride;
-    for (int idx = tid; idx < a.nq * a.D; idx += blockDim.x) {
+    const int first = blockIdx.y * blockDim.x + tid, stride = blockDim.x * gridDim.y;
+    for (int idx = first; idx < a.nq * a.D; idx += stride) {
         const int hd = idx / a.D, c = idx % a.D;
         qrow[idx] = from_f32<TX>(c < a.d ? prepared(0, hd, c, inv_q, wq) : 0.f);
     }
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
     const int page = pi < a.bt_width ? block_table[static_cast<int64_t>(token_entry[t]) * a.bt_width + pi] : -1;
     if (page < 0 || page >= a.num_pages) return;   // no page: the step's host checks make this unreachable
     const int slot = pos % a.page_size;
-    for (int idx = tid; idx < a.nkv * a.D; idx += blockDim.x) {
+    for (int idx = first; idx < a.nkv * a.D; idx += stride) {
         const int g = idx / a.D, c = idx % a.D;
         const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
         kcache[(pg * a.page_size + slot) * a.D + c] = from_f32<TC>(c < a.d ? prepared(nqd, g, c, inv_k, wk) : 0.f);
@@ -139,13 +141,14 @@ extern "C" int pulse_qkv_rows(const void* x, int x_dtype, int64_t x_stride, cons
     const size_t lds = sizeof(float) * (static_cast<size_t>(nq) * d + static_cast<size_t>(nkv) * d);
     PULSE_REQUIRE(lds <= 60 * 1024, "qkv_rows: a token's q and k (%zu bytes in float32) do not fit the workgroup's memory", lds);
     if (tokens == 0) return 0;
+    const int parts = tokens >= 512 ? 1 : min(16, (nq * D + 511) / 512);
     PrepArgs a;
     a.nq = nq; a.nkv = nkv; a.d = d; a.dv = dv; a.D = D; a.x_stride = x_stride; a.q_stride = q_stride;
     a.norm = norm; a.eps = eps; a.rotary_dim = cos_t ? rotary_dim : 0; a.pairing = pairing;
     a.page_size = page_size; a.num_pages = num_pages; a.bt_width = bt_width; a.write_kv = write_kv;
     a.value_scale = value_scale;
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(c_dtype, TC,
-        hipLaunchKernelGGL((qkv_rows_kernel<TX, TW, TC>), dim3(tokens), dim3(256), lds, stream,
+        hipLaunchKernelGGL((qkv_rows_kernel<TX, TW, TC>), dim3(tokens, parts), dim3(256), lds, stream,
                            static_cast<const TX*>(x), static_cast<const TW*>(bq), static_cast<const TW*>(bk),
                            static_cast<const TW*>(bv), static_cast<const TW*>(wq), static_cast<const TW*>(wk), cos_t,
                            sin_t, static_cast<TX*>(q_out), static_cast<TC*>(kcache), static_cast<TC*>(vcache), positions,

@@ -711,11 +711,14 @@ def lightning_row_groups(entries: int, heads: int, d: int, dv: int) -> int:
     """Over how many lanes ``lightning_scan`` shares a column's rows out: the fewest (1, 4, 16) that give the launch
     about as many wavefronts as the chip has places for."""
     from .device import compute_units
-    want = 4 * compute_units()
-    for r in (1, 4, 16):
+    want = 8 * compute_units()
+    # (a workgroup's four wavefronts own 256 columns when a lane holds a whole column: narrower heads would leave
+    # wavefronts idle, so they start at 4 lanes a column)
+    choices = (1, 4, 16) if dv >= 256 else (4, 16)
+    for r in choices:
         if r == 16 and d <= 32:
             break
-        if entries * heads * ((dv * r + 63) // 64) >= want:
+        if entries * heads * ((dv * r + 255) // 256) * 4 >= want:
             return r
     return 16 if d > 32 else 4
 
@@ -723,9 +726,15 @@ def lightning_row_groups(entries: int, heads: int, d: int, dv: int) -> int:
 def lightning_scan(x: torch.Tensor, q0: int, k0: int, v0: int, out: torch.Tensor, state: torch.Tensor,
                    decay: torch.Tensor, entry_first_row: torch.Tensor, entry_start: torch.Tensor,
                    entry_slot: torch.Tensor, heads: int, d: int, dv: int, activation: str = "silu",
-                   row_groups: int = 1) -> None:
+                   row_groups: int = 1, pieces: Optional[torch.Tensor] = None,
+                   scratch: Optional[torch.Tensor] = None) -> None:
     """For every entry of the step, token by token: S <- decay_h S + k v^T, out = S^T q, per head, in float32;
-    S [slots, heads, d, dv] is the state of the entry's slot, zero when the entry starts at position 0."""
+    S [slots, heads, d, dv] is the state of the entry's slot, zero when the entry starts at position 0.
+
+    ``pieces`` (int32 [n, 4]: first row, tokens, entry, 1 for an entry's first piece | 2 for its last; an entry's
+    pieces in order and next to each other) with ``scratch`` (float32 [n, heads, d, dv]): the entries are walked in
+    these pieces, all at the same time: every piece from a zero state, then the states between the pieces from what
+    each left, then every piece again with its outputs."""
     _gpu("lightning_scan", x, out, state, decay, entry_first_row, entry_start, entry_slot)
     entries = entry_start.numel()
     _need(x.dim() == 2 and x.stride(1) == 1, "lightning_scan: x must be a matrix with contiguous rows")
@@ -742,10 +751,40 @@ def lightning_scan(x: torch.Tensor, q0: int, k0: int, v0: int, out: torch.Tensor
     width = x.shape[1]
     _need(min(q0, k0, v0) >= 0 and max(q0, k0) + heads * d <= width and v0 + heads * dv <= width,
           "lightning_scan: q, k or v columns lie outside x")
-    call("pulse_lightning_scan", _ptr(x), _i32(_tag(x, "lightning_scan")), _i64(x.stride(0)), _i32(q0), _i32(k0), _i32(v0),
-         _ptr(out), _i64(out.stride(0)), _ptr(state), _i32(state.shape[0]), _ptr(decay), _ptr(entry_first_row),
-         _ptr(entry_start), _ptr(entry_slot), _i32(entries), _i32(heads), _i32(d), _i32(dv),
-         _i32(1 if activation == "silu" else 0), _i32(row_groups), _stream())
+    def walk(mode: int, n_pieces: int) -> None:
+        call("pulse_lightning_scan", _ptr(x), _i32(_tag(x, "lightning_scan")), _i64(x.stride(0)), _i32(q0), _i32(k0),
+             _i32(v0), _ptr(out), _i64(out.stride(0)), _ptr(state), _i32(state.shape[0]), _ptr(decay),
+             _ptr(entry_first_row), _ptr(entry_start), _ptr(entry_slot), _i32(entries), _i32(heads), _i32(d), _i32(dv),
+             _i32(1 if activation == "silu" else 0), _i32(row_groups), _i32(mode), _ptr(pieces), _i32(n_pieces),
+             _ptr(scratch), _stream())
+
+    if pieces is None:
+        walk(0, 0)
+        return
+    _gpu("lightning_scan", pieces, scratch)
+    n_pieces = pieces.numel() // 4
+    _need(pieces.dtype == torch.int32 and pieces.is_contiguous() and pieces.numel() == 4 * n_pieces and n_pieces > 0,
+          "lightning_scan: pieces must be int32 quadruples")
+    _need(scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous()
+          and scratch.numel() >= n_pieces * heads * d * dv, "lightning_scan: the scratch for the pieces' states is too small")
+    walk(1, n_pieces)
+    call("pulse_lightning_combine", _ptr(scratch), _ptr(state), _ptr(decay), _ptr(pieces), _i32(n_pieces), _ptr(entry_start),
+         _ptr(entry_slot), _i32(heads), _i32(d), _i32(dv), _stream())
+    walk(2, n_pieces)
+
+
+def lightning_pieces(entries, piece_tokens: int):
+    """The step's entries cut into pieces of ``piece_tokens`` tokens for ``lightning_scan`` (flat quadruples), or None
+    when no entry is long enough for the walk in pieces to pay (twice ``piece_tokens``)."""
+    if not any(e.count >= 2 * piece_tokens for e in entries):
+        return None
+    flat = []
+    for index, e in enumerate(entries):
+        cuts = list(range(0, e.count, piece_tokens)) if e.count >= 2 * piece_tokens else [0]
+        for j, at in enumerate(cuts):
+            end = cuts[j + 1] if j + 1 < len(cuts) else e.count
+            flat.extend((e.first_row + at, end - at, index, (1 if j == 0 else 0) | (2 if j + 1 == len(cuts) else 0)))
+    return flat
 
 
 def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, eps: float,
@@ -782,6 +821,25 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
           f"moe_route: idx int32 and weight float32 must be [{tokens}, {top}]")
     call("pulse_moe_route", _ptr(logits), _ptr(correction), _i32(_tag(correction, "moe_route") if correction is not None else 0),
          _ptr(idx), _ptr(weight), _i32(tokens), _i32(n), _i32(top), _stream())
+
+
+def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
+               weight: torch.Tensor) -> None:
+    """``moe_route`` of the logits x w_router^T, which are formed in float32 inside the kernel."""
+    _gpu("moe_router", x, w_router, correction, idx, weight)
+    tokens, hidden = x.shape
+    n = w_router.shape[0]
+    _need(x.is_contiguous() and w_router.is_contiguous() and w_router.shape[1] == hidden,
+          f"moe_router: x [T, {hidden}] and the router's weight [outputs, {hidden}] must be contiguous")
+    _need(correction is None or (correction.numel() == n and correction.is_contiguous()
+                                 and correction.dtype == w_router.dtype),
+          f"moe_router: the correction must hold {n} values of the weight's storage type")
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and tuple(idx.shape) == (tokens, top)
+          and weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == (tokens, top),
+          f"moe_router: idx int32 and weight float32 must be [{tokens}, {top}]")
+    call("pulse_moe_router", _ptr(x), _i32(_tag(x, "moe_router")), _ptr(w_router), _ptr(correction),
+         _i32(_tag(w_router, "moe_router")), _ptr(idx), _ptr(weight), _i32(tokens), _i32(hidden), _i32(n), _i32(top),
+         _stream())
 
 
 def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor) -> None:

@@ -107,9 +107,21 @@ class LightningAttention(Part):
         y = ws.buffer("lightning.proj", tokens, 2 * hd + 2 * hv, self.act_dtype)
         self.proj.forward(x, y)
         o = ws.buffer("lightning.heads", tokens, hv, torch.float32)
-        groups = kernels.lightning_row_groups(len(ctx.entries), self.heads, self.d, self.dv)
+        # long portions are walked in pieces that run at the same time (the list depends on the step's shape alone)
+        piece_tokens = 64 if tokens < 1024 else 128
+        key = f"static:lightning.pieces:{piece_tokens}"
+        if key not in ctx.extras:
+            flat = kernels.lightning_pieces(ctx.entries, piece_tokens)
+            ctx.extras[key] = ctx.to_device(flat) if flat else None
+        pieces = ctx.extras[key]
+        scratch = None
+        walkers = len(ctx.entries)
+        if pieces is not None:
+            walkers = pieces.numel() // 4
+            scratch = ws.buffer("lightning.pieces", walkers, self.heads * self.d * self.dv, torch.float32)
+        groups = kernels.lightning_row_groups(walkers, self.heads, self.d, self.dv)
         kernels.lightning_scan(y, 0, hd, 2 * hd, o, cache.state, self.decay, ctx.entry_first_row, ctx.entry_start,
-                               ctx.entry_slot, self.heads, self.d, self.dv, self.activation, groups)
+                               ctx.entry_slot, self.heads, self.d, self.dv, self.activation, groups, pieces, scratch)
         kernels.gated_rmsnorm(o, self.norm_weight, y[:, 2 * hd + hv:], out, self.eps, self.out_scale)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: StateView) -> torch.Tensor:

@@ -95,6 +95,8 @@ class RoutedExperts(Part):
         n = self.tensor_names(params)
         self.router = load.get(joined(prefix, n["router"]))
         self.correction = load.get(joined(prefix, n["correction"])) if params.get("correction", False) else None
+        if self.correction is not None and self.correction.dtype != self.router.dtype:
+            self.correction = self.correction.to(self.router.dtype)
         stack = lambda which: torch.stack([load.get(joined(joined(prefix, n["expert"].format(e=e)), n[which]))
                                            for e in range(self.experts)], dim=0).contiguous()
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
@@ -109,12 +111,9 @@ class RoutedExperts(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext):
         tokens = x.shape[0]
         ws = ctx.workspace
-        outputs = self.experts + self.identity
-        z = ws.buffer("moe.logits", tokens, outputs, torch.float32)
-        kernels.gemm_f32(x, self.router, z)
         idx = ws.buffer("moe.idx", tokens, self.top, torch.int32)
         weight = ws.buffer("moe.weight", tokens, self.top, torch.float32)
-        kernels.moe_route(z, self.correction, self.top, idx, weight)
+        kernels.moe_router(x, self.router, self.correction, self.top, idx, weight)   # logits in float32 inside
         act = ws.buffer("moe.act", tokens * self.top, self.ff, self.act_dtype)
         routed = ws.buffer("moe.out", tokens, self.hidden, torch.float32)
         if kernels.moe_grouped_takes(x, self.w_gate, self.w_down):

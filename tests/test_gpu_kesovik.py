@@ -215,6 +215,57 @@ def test_the_state_walk(dtype, heads, d, dv, groups):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,d,dv,groups,piece", [(3, 16, 32, 1, 16), (2, 64, 64, 16, 32), (4, 128, 128, 4, 64),
+                                                     (1, 48, 100, 4, 16)])
+def test_the_state_walk_in_pieces(dtype, heads, d, dv, groups, piece):
+    """A long portion that continues a state, a fresh one, a short one and a single token in one step, the long ones
+    cut into pieces that are walked at the same time: outputs and final states are those of the walk token by token,
+    and of the plain walk."""
+    from pulse_infer_amd.ops import kernels
+
+    class E:
+        def __init__(self, first_row, count):
+            self.first_row, self.count = first_row, count
+
+    decay = [0.5, 1.0, 0.97, 0.999][:heads]
+    counts, starts, slot_of = [5 * piece + 3, 2 * piece, piece + 1, 1], [7, 0, 40, 300], [3, 0, 4, 1]
+    first = [0]
+    for n in counts:
+        first.append(first[-1] + n)
+    flat = kernels.lightning_pieces([E(f, n) for f, n in zip(first, counts)], piece)
+    assert flat is not None and len(flat) // 4 == 6 + 2 + 1 + 1
+    state = torch.full((5, heads, d, dv), float("nan"), device=DEV)
+    before = {}
+    for i, slot in enumerate(slot_of):
+        if starts[i]:
+            before[i] = rnd(heads, d, dv, seed=40 + i)
+            state[slot] = before[i].to(DEV)
+    whole = state.clone()
+    cols = 2 * heads * d + heads * dv
+    lam = torch.tensor(decay, dtype=torch.float32, device=DEV)
+    x, xref = stored(rnd(first[-1], cols, seed=9), dtype)
+    out = torch.full((first[-1], heads * dv), float("nan"), device=DEV)
+    scratch = torch.full((len(flat) // 4, heads, d, dv), float("nan"), device=DEV)
+    kernels.lightning_scan(x, 0, heads * d, 2 * heads * d, out, state, lam, ints(first), ints(starts), ints(slot_of),
+                           heads, d, dv, "silu", groups, ints(flat), scratch)
+    direct = torch.full_like(out, float("nan"))
+    kernels.lightning_scan(x, 0, heads * d, 2 * heads * d, direct, whole, lam, ints(first), ints(starts), ints(slot_of),
+                           heads, d, dv, "silu", groups)
+    for i in range(len(counts)):
+        rows = xref[first[i]:first[i + 1]]
+        q = P.silu(rows[:, :heads * d]).view(-1, heads, d)
+        k = P.silu(rows[:, heads * d:2 * heads * d]).view(-1, heads, d)
+        v = P.silu(rows[:, 2 * heads * d:]).view(-1, heads, dv)
+        want, last = P.decayed_state_walk(q, k, v, decay, before[i].to(F64) if starts[i] else None)
+        got = out[first[i]:first[i + 1]].cpu().to(F64).view(-1, heads, dv)
+        scale = max(1.0, float(want.abs().max()))
+        assert float((got - want).abs().max()) <= 5e-5 * scale, i
+        assert float((got - direct[first[i]:first[i + 1]].cpu().to(F64).view(-1, heads, dv)).abs().max()) <= 5e-5 * scale
+        assert float((state[slot_of[i]].cpu().to(F64) - last).abs().max()) <= 5e-5 * max(1.0, float(last.abs().max()))
+    assert torch.isnan(state[2]).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_heads_normed_together_and_gated(dtype):
     from pulse_infer_amd.ops import kernels
 
@@ -398,6 +449,9 @@ def test_router_and_experts(dtype, experts, identity, top, ff, hidden):
     assert torch.allclose(weight.cpu().to(F64), want_w, atol=1e-5)
     if identity:
         assert int((want_idx >= experts).sum()) > 0
+    idx2, weight2 = torch.full_like(idx, -7), torch.full_like(weight, float("nan"))
+    kernels.moe_router(x, router, corr, top, idx2, weight2)          # product and routing in one kernel
+    assert torch.equal(idx2, idx) and torch.allclose(weight2, weight, atol=1e-5)
     wg, gref = stored(rnd(experts, ff, hidden, seed=4, scale=hidden ** -0.5), dtype)
     wu, uref = stored(rnd(experts, ff, hidden, seed=5, scale=hidden ** -0.5), dtype)
     wd, dref = stored(rnd(experts, hidden, ff, seed=6, scale=ff ** -0.5), dtype)
