@@ -659,6 +659,77 @@ def test_a_long_prompt_far_beyond_the_windows(runners, plain, dtype):
     agree(run_alone(runner, ids, [150, 190] + [1] * 60), want, dtype, "decoded tail", calls)
 
 
+# ------------------------------------------------------------------------------------ seeded random configurations
+def random_config(rng):
+    """Layers drawn one by one: head sizes that are no multiples of 16, keys wider or narrower than values, any
+    grouping of heads, windows from one token on, rotations on a part of a head, inner widths that are no multiples of
+    8 (the experts' products then take the kernel without matrix cores), routers that choose all their outputs."""
+    width = rng.choice([64, 96, 160, 256])
+    layers = []
+    for _ in range(rng.choice([1, 2, 3])):
+        heads = rng.choice([1, 2, 3, 5])
+        light = lightning(heads, rng.choice([16, 24, 32, 64]), rng.choice([16, 20, 32, 72]),
+                          [rng.choice([0.0, 0.5, 0.9, 0.99, 1.0]) for _ in range(heads)])
+        if rng.random() < 0.6:
+            groups, share = rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 4])
+            dim = rng.choice([16, 24, 32, 48, 64])
+            rot = rng.choice([d for d in (2, 8, 16, 24, dim) if d <= dim])
+            mixer = parallel(left(groups * share, groups, dim, rng.choice([8, 16, 40, 48, 64]), rng.choice([1, 5, 16, 33, 100]),
+                                  rot, rng.choice([100.0, 1e4, 5e5]), rng.choice([0.1, dim ** -0.5, 0.5])),
+                             light, rng.choice([0.5, 1.0, 1.5]), rng.choice([0.7, 1.0]))
+        else:
+            mixer = light
+        kind = rng.choice(["none", "dense", "moe", "moe"])
+        if kind == "none":
+            mlp = None
+        elif kind == "dense":
+            mlp = dense(rng.choice([32, 100, 256]))
+        else:
+            experts, identity = rng.choice([1, 2, 4, 9]), rng.choice([0, 1, 3])
+            mlp = moe(experts, identity, rng.randint(1, min(4, experts + identity)), rng.choice([32, 40, 64, 100]),
+                      rng.choice([None, 48, 128]))
+        layers.append(layer(mixer, mlp))
+    return config(rng.choice([257, 300, 1000]), width, rng.choice([1e-6, 1e-5]), rng.choice([1.0, 2.5, 4.0]),
+                  rng.choice([1.0, 3.0]), rng.choice([5.0, 15.0, 50.0]), layers)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(tmp_path, seed):
+    """Whole, with the last 20 tokens one by one, and in portions of 2 to 70 tokens, in 32-bit and in bfloat16."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    import random
+
+    from pulse_infer_amd.config import KesovikConfig
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    rng = random.Random(7000 + seed)
+    cfg = random_config(rng)
+    length = rng.choice([90, 150])
+    folder = write_model_folder(KesovikConfig.from_dict(cfg), str(tmp_path / "m"), seed=seed)
+    oracle = P.PlainKesovik.from_folder(folder)
+    ids = token_ids(cfg["vocab"], length, seed=seed)
+    want = oracle.logits(ids)
+    calls = set((oracle.router_margins(ids) < CLOSE_CALL).nonzero().flatten().tolist())
+    what = f"{cfg} length {length}"
+    for dtype in ("float32", "bfloat16"):
+        _, model = load_model(folder, mode=dtype)
+        runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=4)
+        whole = run_alone(runner, ids, [length])
+        agree(whole, want, dtype, f"whole: {what}", calls)
+        agree(run_alone(runner, ids, [length - 20] + [1] * 20), want, dtype, f"tail: {what}", calls)
+        cuts, left_over, sizes = [], length, [40, 2, 17, 3, 70, 5, 19]
+        while left_over:
+            n = min(sizes[len(cuts) % len(sizes)], left_over)
+            cuts.append(n)
+            left_over -= n
+        agree(run_alone(runner, ids, cuts), want, dtype, f"portions {cuts}: {what}", calls)
+        del runner, model
+    torch.cuda.empty_cache()
+
+
 # ------------------------------------------------------------------------------------------------ long decoding
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["mixed", "wide"])
