@@ -232,11 +232,13 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, int64_t o_stri
     const int t = blockIdx.x;
     const float* row = o + static_cast<int64_t>(t) * o_stride;
     float ss = 0.f;
+#pragma unroll 4
     for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(row[i], row[i], ss);
     const float total = block_sum(ss, scratch);
     const float inv = scale / sqrtf(total / static_cast<float>(n) + eps);
     const TX* g = gate ? gate + static_cast<int64_t>(t) * gate_stride : nullptr;
     TX* dst = y + static_cast<int64_t>(t) * y_stride;
+#pragma unroll 4
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = row[i] * inv * to_f32<TW>(w[i]);
         if (g) v *= 1.0f / (1.0f + expf(-to_f32<TX>(g[i])));

@@ -92,20 +92,22 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
 // take the router's outputs in turn (float32 multiply-adds over the hidden size, lanes sharing a dot product out),
 // and the first wavefront routes.
 template <typename TX, typename TW>
-__global__ __launch_bounds__(256) void moe_router_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
+__global__ __launch_bounds__(1024) void moe_router_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
                                                          const TW* __restrict__ correction, int* __restrict__ idx,
                                                          float* __restrict__ weight, int hidden, int n, int top) {
     extern __shared__ float x_s[];          // [hidden] then [n]
     float* z_s = x_s + hidden;
     const int t = blockIdx.x;
+#pragma unroll 4
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) x_s[i] = to_f32<TX>(x[static_cast<int64_t>(t) * hidden + i]);
     __syncthreads();
-    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE, waves = blockDim.x / PULSE_WAVE;
     const bool wide = sizeof(TW) == 2 && hidden % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
-    for (int o = wave; o < n; o += 4) {
+    for (int o = wave; o < n; o += waves) {
         const TW* wrow = w + static_cast<int64_t>(o) * hidden;
         float sum = 0.f;
         if (wide) {   // 16 bytes of a bfloat16 row a lane and step
+#pragma unroll 4
             for (int i = lane * 8; i < hidden; i += PULSE_WAVE * 8) {
                 const pulse_i32x4 raw = *reinterpret_cast<const pulse_i32x4*>(wrow + i);
 #pragma unroll
@@ -215,7 +217,8 @@ extern "C" int pulse_moe_router(const void* x, int x_dtype, const void* w, const
     PULSE_REQUIRE(lds <= 60 * 1024, "moe_router: rows of %d values do not fit the workgroup's memory", hidden);
     if (tokens == 0) return 0;
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
-        hipLaunchKernelGGL((moe_router_kernel<TX, TW>), dim3(tokens), dim3(256), lds, stream, static_cast<const TX*>(x),
+        hipLaunchKernelGGL((moe_router_kernel<TX, TW>), dim3(tokens), dim3(tokens <= 256 ? 1024 : 256), lds, stream,
+                           static_cast<const TX*>(x),
                            static_cast<const TW*>(w), static_cast<const TW*>(correction), idx, weight, hidden, n, top)));
     PULSE_LAUNCH_CHECK("moe_router");
     return 0;

@@ -74,24 +74,60 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int* __r
     }
 }
 
+// Tiles of 32 rows (decoding: few rows an expert) give few workgroups, each with a long walk: there the four
+// wavefronts of a workgroup own the SAME 16 weight rows and a quarter of the k-steps each, and their sums meet in LDS in
+// wavefront order (four times the workgroups, four times the loads in flight, the same result from run to run).
+template <int NW, int RB>
+__device__ __forceinline__ bool meet(f32x4 (&acc)[NW][RB], float* red, int wave, int lane) {
+    // red: [4][NW * RB][64][4] floats
+#pragma unroll
+    for (int s = 0; s < NW; ++s)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((wave * NW * RB + s * RB + rb) * 64 + lane) * 4 + i] = acc[s][rb][i];
+    __syncthreads();
+    if (wave != 0) return false;
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+#pragma unroll
+        for (int s = 0; s < NW; ++s)
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[s][rb][i] += red[((w * NW * RB + s * RB + rb) * 64 + lane) * 4 + i];
+    return true;
+}
+
 // One tile of one expert against 64 weight rows: acc[rb] += W[16 rows of this wavefront] . X[16 rows of block rb]^T.
 // wrow: this lane's weight row (null: beyond the weight), xrow[rb]: this lane's row of block rb (null: no such row).
 template <int RB, int NW>
 __device__ __forceinline__ void walk(const bf16_t* const (&wrow)[NW], const bf16_t* const (&xrow)[RB], int blocks, int K,
-                                     int kg, f32x4 (&acc)[NW][RB]) {
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        const int kc = k0 + kg * 8;
-        const bool kok = kc < K;   // K is a multiple of 8
-        bf16x8 wa[NW];
+                                     int kg, f32x4 (&acc)[NW][RB], int share = 0, int shares = 1) {
+    constexpr int U = 4;   // k-steps whose loads are asked for before the first of them is used
+    // (`share` of `shares`: this wavefront takes every shares-th group of U k-steps, from group `share` on)
+    for (int k0 = share * 32 * U; k0 < K; k0 += shares * 32 * U) {
+        bf16x8 wa[U][NW], xb[U][RB];
 #pragma unroll
-        for (int s = 0; s < NW; ++s)
-            wa[s] = (kok && wrow[s]) ? *reinterpret_cast<const bf16x8*>(wrow[s] + kc) : zeros8();
+        for (int u = 0; u < U; ++u) {
+            const int kc = k0 + 32 * u + kg * 8;
+            const bool kok = kc < K;   // K is a multiple of 8
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            if (rb < blocks) {
-                const bf16x8 xb = (kok && xrow[rb]) ? *reinterpret_cast<const bf16x8*>(xrow[rb] + kc) : zeros8();
+            for (int s = 0; s < NW; ++s)
+                wa[u][s] = (kok && wrow[s]) ? *reinterpret_cast<const bf16x8*>(wrow[s] + kc) : zeros8();
 #pragma unroll
-                for (int s = 0; s < NW; ++s) acc[s][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[s], xb, acc[s][rb], 0, 0, 0);
+            for (int rb = 0; rb < RB; ++rb)
+                xb[u][rb] = (kok && rb < blocks && xrow[rb]) ? *reinterpret_cast<const bf16x8*>(xrow[rb] + kc) : zeros8();
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                if (rb < blocks) {
+#pragma unroll
+                    for (int s = 0; s < NW; ++s)
+                        acc[s][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][s], xb[u][rb], acc[s][rb], 0, 0, 0);
+                }
             }
         }
     }
@@ -159,7 +195,9 @@ __global__ __launch_bounds__(256) void moe_gate_up_grouped_kernel(const bf16_t* 
     const int e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];
     const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
     const int r = lane % 16, kg = lane / 16;
-    const int n = blockIdx.y * 64 + wave * 16 + r;
+    constexpr bool SHARED_K = RB == 2;
+    const int n0 = SHARED_K ? blockIdx.y * 16 : blockIdx.y * 64 + wave * 16;
+    const int n = n0 + r;
     const bf16_t* wrow[2];
     wrow[0] = n < ff ? wg + (static_cast<int64_t>(e) * ff + n) * hidden : nullptr;
     wrow[1] = n < ff ? wu + (static_cast<int64_t>(e) * ff + n) * hidden : nullptr;
@@ -183,10 +221,12 @@ __global__ __launch_bounds__(256) void moe_gate_up_grouped_kernel(const bf16_t* 
         walk_staged<2>(wrow, p >= 0 ? x + static_cast<int64_t>(p / top) * hidden : nullptr, stage, (rows + 15) / 16, hidden,
                        r, kg, acc);
     } else {
-        walk<RB, 2>(wrow, xrow, (rows + 15) / 16, hidden, kg, acc);
+        __shared__ float red[4 * 2 * RB * 64 * 4];
+        walk<RB, 2>(wrow, xrow, (rows + 15) / 16, hidden, kg, acc, wave, 4);
+        if (!meet<2, RB>(acc, red, wave, lane)) return;
     }
     // lane l holds inner columns 4 * (l / 16) + i of this wavefront's 16, for row l % 16 of every block
-    const int j0 = blockIdx.y * 64 + wave * 16 + 4 * kg;
+    const int j0 = n0 + 4 * kg;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
         if (pair[rb] < 0) continue;
@@ -215,7 +255,9 @@ __global__ __launch_bounds__(256) void moe_down_grouped_kernel(const bf16_t* __r
     const int e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];
     const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
     const int r = lane % 16, kg = lane / 16;
-    const int n = blockIdx.y * 64 + wave * 16 + r;
+    constexpr bool SHARED_K = RB == 2;
+    const int n0 = SHARED_K ? blockIdx.y * 16 : blockIdx.y * 64 + wave * 16;
+    const int n = n0 + r;
     const bf16_t* wrow[1];
     wrow[0] = n < hidden ? wd + (static_cast<int64_t>(e) * hidden + n) * ff : nullptr;
     const bf16_t* xrow[RB];
@@ -235,9 +277,11 @@ __global__ __launch_bounds__(256) void moe_down_grouped_kernel(const bf16_t* __r
         const int p = mine < rows ? order[row0 + mine] : -1;
         walk_staged<1>(wrow, p >= 0 ? act + static_cast<int64_t>(p) * ff : nullptr, stage, (rows + 15) / 16, ff, r, kg, acc);
     } else {
-        walk<RB, 1>(wrow, xrow, (rows + 15) / 16, ff, kg, acc);
+        __shared__ float red[4 * 1 * RB * 64 * 4];
+        walk<RB, 1>(wrow, xrow, (rows + 15) / 16, ff, kg, acc, wave, 4);
+        if (!meet<1, RB>(acc, red, wave, lane)) return;
     }
-    const int c0 = blockIdx.y * 64 + wave * 16 + 4 * kg;
+    const int c0 = n0 + 4 * kg;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
         if (pair[rb] < 0) continue;
@@ -295,10 +339,10 @@ extern "C" int pulse_moe_gate_up_grouped(const void* x, const void* wg, const vo
     PULSE_REQUIRE(tile_rows_max == 32 || tile_rows_max == 128, "moe_gate_up_grouped: tiles of 32 or 128 rows");
     PULSE_REQUIRE(x && wg && wu && order && tile_expert && tile_row0 && tile_rows && num_tiles && act,
                   "moe_gate_up_grouped: null pointer");
-    PULSE_REQUIRE((ff + 63) / 64 < 65536, "moe_gate_up_grouped: an inner width of %d is too large", ff);
+    PULSE_REQUIRE((ff + 15) / 16 < 65536, "moe_gate_up_grouped: an inner width of %d is too large", ff);
     const dim3 grid(max_tiles, (ff + 63) / 64);
     if (tile_rows_max == 32)
-        hipLaunchKernelGGL(moe_gate_up_grouped_kernel<2>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x),
+        hipLaunchKernelGGL(moe_gate_up_grouped_kernel<2>, dim3(max_tiles, (ff + 15) / 16), dim3(256), 0, stream, static_cast<const bf16_t*>(x),
                            static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(wu), order, tile_expert, tile_row0,
                            tile_rows, num_tiles, static_cast<bf16_t*>(act), hidden, ff, top);
     else
@@ -318,10 +362,10 @@ extern "C" int pulse_moe_down_grouped(const void* act, const void* wd, const int
     PULSE_REQUIRE(tile_rows_max == 32 || tile_rows_max == 128, "moe_down_grouped: tiles of 32 or 128 rows");
     PULSE_REQUIRE(act && wd && order && tile_expert && tile_row0 && tile_rows && num_tiles && y,
                   "moe_down_grouped: null pointer");
-    PULSE_REQUIRE((hidden + 63) / 64 < 65536, "moe_down_grouped: a width of %d is too large", hidden);
+    PULSE_REQUIRE((hidden + 15) / 16 < 65536, "moe_down_grouped: a width of %d is too large", hidden);
     const dim3 grid(max_tiles, (hidden + 63) / 64);
     if (tile_rows_max == 32)
-        hipLaunchKernelGGL(moe_down_grouped_kernel<2>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(act),
+        hipLaunchKernelGGL(moe_down_grouped_kernel<2>, dim3(max_tiles, (hidden + 15) / 16), dim3(256), 0, stream, static_cast<const bf16_t*>(act),
                            static_cast<const bf16_t*>(wd), order, tile_expert, tile_row0, tile_rows, num_tiles, y, hidden, ff);
     else
         hipLaunchKernelGGL(moe_down_grouped_kernel<8>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(act),

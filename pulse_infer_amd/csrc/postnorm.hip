@@ -22,6 +22,7 @@ __global__ void scale_add_rmsnorm_kernel(float* __restrict__ h, const T1* __rest
     const int64_t r = blockIdx.x;
     float* hrow = h + r * hidden;
     float ss = 0.f;
+#pragma unroll 4
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = alpha * hrow[i];
         float d = 0.f;
@@ -33,6 +34,7 @@ __global__ void scale_add_rmsnorm_kernel(float* __restrict__ h, const T1* __rest
         ss = fmaf(v, v, ss);
     }
     const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(hidden) + eps);
+#pragma unroll 4
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         const float y = row_s[i] * inv * to_f32<TW>(w[i]);
         hrow[i] = y;

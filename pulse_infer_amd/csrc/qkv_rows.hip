@@ -48,6 +48,7 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
     const int nqd = a.nq * a.d, nkd = a.nkv * a.d, nvd = a.nkv * a.dv;
     const TX* row = x + static_cast<int64_t>(t) * a.x_stride;
     float sq = 0.f, sk = 0.f;
+#pragma unroll 4
     for (int i = tid; i < nqd; i += blockDim.x) {
         float v = to_f32<TX>(row[i]);
         if (bq) v += to_f32<TW>(bq[i]);
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
         sq = fmaf(v, v, sq);
     }
     if (a.write_kv) {
+#pragma unroll 4
         for (int i = tid; i < nkd; i += blockDim.x) {
             float v = to_f32<TX>(row[nqd + i]);
             if (bk) v += to_f32<TW>(bk[i]);
@@ -92,6 +94,7 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
     };
     TX* qrow = q_out + static_cast<int64_t>(t) * a.q_stride;
     const int first = blockIdx.y * blockDim.x + tid, stride = blockDim.x * gridDim.y;
+#pragma unroll 4
     for (int idx = first; idx < a.nq * a.D; idx += stride) {
         const int hd = idx / a.D, c = idx % a.D;
         qrow[idx] = from_f32<TX>(c < a.d ? prepared(0, hd, c, inv_q, wq) : 0.f);
@@ -102,19 +105,45 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
     const int page = pi < a.bt_width ? block_table[static_cast<int64_t>(token_entry[t]) * a.bt_width + pi] : -1;
     if (page < 0 || page >= a.num_pages) return;   // no page: the step's host checks make this unreachable
     const int slot = pos % a.page_size;
+#pragma unroll 2
     for (int idx = first; idx < a.nkv * a.D; idx += stride) {
         const int g = idx / a.D, c = idx % a.D;
         const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
         kcache[(pg * a.page_size + slot) * a.D + c] = from_f32<TC>(c < a.d ? prepared(nqd, g, c, inv_k, wk) : 0.f);
+    }
+    (void)nvd;
+    (void)bv;
+    (void)vcache;
+}
+
+// The values go to their pages from a kernel of their own: a page holds a channel's slots side by side, so a
+// workgroup takes 16 consecutive tokens and one key/value head, a token a lane of every group of 16 lanes: the 16
+// lanes of a group then fill neighbouring slots of one channel (32 contiguous bytes in bfloat16) where a token at a
+// time would write two-byte pieces a whole page row apart.
+template <typename TX, typename TW, typename TC>
+__global__ __launch_bounds__(256) void v_rows_kernel(const TX* __restrict__ x, const TW* __restrict__ bv,
+                                                     TC* __restrict__ vcache, const int* __restrict__ positions,
+                                                     const int* __restrict__ token_entry,
+                                                     const int* __restrict__ block_table, int tokens, PrepArgs a) {
+    const int tt = threadIdx.x % 16, cc = threadIdx.x / 16;
+    const int t = blockIdx.x * 16 + tt, g = blockIdx.y;
+    if (t >= tokens) return;
+    const int pos = positions[t];
+    const int pi = pos / a.page_size;
+    const int page = pi < a.bt_width ? block_table[static_cast<int64_t>(token_entry[t]) * a.bt_width + pi] : -1;
+    if (page < 0 || page >= a.num_pages) return;
+    const int slot = pos % a.page_size;
+    const TX* src = x + static_cast<int64_t>(t) * a.x_stride + a.nq * a.d + a.nkv * a.d + g * a.dv;
+    TC* dst = vcache + (static_cast<int64_t>(page) * a.nkv + g) * a.D * a.page_size + slot;
+    for (int c = cc; c < a.D; c += 16) {
         float v = 0.f;
         if (c < a.dv) {
-            v = to_f32<TX>(row[nqd + nkd + g * a.dv + c]);
+            v = to_f32<TX>(src[c]);
             if (bv) v += to_f32<TW>(bv[g * a.dv + c]);
             v *= a.value_scale;
         }
-        vcache[(pg * a.D + c) * a.page_size + slot] = from_f32<TC>(v);
+        dst[static_cast<int64_t>(c) * a.page_size] = from_f32<TC>(v);
     }
-    (void)nvd;
 }
 
 }  // namespace
@@ -154,5 +183,13 @@ extern "C" int pulse_qkv_rows(const void* x, int x_dtype, int64_t x_stride, cons
                            sin_t, static_cast<TX*>(q_out), static_cast<TC*>(kcache), static_cast<TC*>(vcache), positions,
                            token_entry, block_table, a))));
     PULSE_LAUNCH_CHECK("qkv_rows");
+    if (write_kv) {
+        PULSE_REQUIRE(nkv < 65536, "qkv_rows: too many key/value heads");
+        PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(c_dtype, TC,
+            hipLaunchKernelGGL((v_rows_kernel<TX, TW, TC>), dim3((tokens + 15) / 16, nkv), dim3(256), 0, stream,
+                               static_cast<const TX*>(x), static_cast<const TW*>(bv), static_cast<TC*>(vcache), positions,
+                               token_entry, block_table, tokens, a))));
+        PULSE_LAUNCH_CHECK("qkv_rows (values)");
+    }
     return 0;
 }
