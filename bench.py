@@ -242,7 +242,7 @@ def kesovik_layers(size, layers):
     def lightning(heads):
         decay = [1.0 - 2.0 ** -(5 + 8.0 * h / heads) for h in range(heads)]
         return {"decay": decay, "dim": size["dim"], "heads": heads, "vdim": size["dim"]}
-    both = {"left": left, "left_scale": 0.8, "right": lightning(size["heads"] // 2), "right_scale": 1.1}
+    both = {"left": left, "left_scale": 0.9, "right": lightning(size["heads"] // 2), "right_scale": 1.2}
     dense = {"ff": size["ff"], "kind": "dense"}
     routed = {"expert": {"ff": size["ff"] // 8}, "kind": "moe", "router": {"experts": 16, "identity": 2, "top": 4},
               "shared": {"ff": size["ff"] // 4}}

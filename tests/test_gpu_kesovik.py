@@ -426,7 +426,7 @@ def test_prepared_rows_and_the_window(case, dtype, needle):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("experts,identity,top,ff,hidden", [(5, 2, 3, 48, 96), (3, 0, 1, 64, 80), (12, 4, 4, 64, 256),
+@pytest.mark.parametrize("experts,identity,top,ff,hidden", [(5, 2, 3, 48, 96), (3, 0, 1, 64, 80), (10, 3, 4, 72, 192),
                                                             (2, 1, 3, 40, 64)])
 def test_router_and_experts(dtype, experts, identity, top, ff, hidden):
     """Choice by score plus correction (a correction large enough to change the choice), weights from the scores
