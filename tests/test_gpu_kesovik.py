@@ -296,7 +296,8 @@ def paged(lens, nkv, d, bs, dtype, seed):
 
 
 WINDOW_CASES = [
-    dict(nq=6, nkv=2, d=32, dv=16, bs=16, window=24, rot=16, lens=[150, 1, 64, 65], portion=70),
+    dict(nq=6, nkv=2, d=32, dv=16, bs=16, window=24, rot=16, lens=[150, 1, 64, 65, 71, 72, 73], portion=70),   # (the
+    # window's far edge of the last three lies at a page's last and first slot)
     dict(nq=4, nkv=4, d=16, dv=48, bs=16, window=7, rot=16, lens=[90, 33, 17], portion=40),
     dict(nq=8, nkv=2, d=128, dv=128, bs=32, window=64, rot=64, lens=[257, 100], portion=129),
     dict(nq=3, nkv=1, d=48, dv=96, bs=16, window=40, rot=48, lens=[200, 41, 40, 5], portion=2),
