@@ -77,34 +77,43 @@ class WindowAttentionSizes:
     dim: int
     vdim: int
     scale: float
-    window: int
+    window: Optional[int]       # None: config.json names no mask, every earlier token is visible
     rot_base: float
-    rot_dims: int
+    rot_dims: int               # 0: config.json names no rotation
 
     @classmethod
     def read(cls, data: Dict[str, Any], where: str) -> "WindowAttentionSizes":
         r = JsonReader(data, where)
-        mask = JsonReader(_object(r.raw("mask"), where, "mask"), f"{where}.mask")
-        rot = JsonReader(_object(r.raw("rot"), where, "rot"), f"{where}.rot")
         dim = r.integer("dim")
-        return cls(heads=r.integer("heads"), kv_heads=r.integer("kv_heads"), dim=dim, vdim=r.integer("vdim", dim),
-                   scale=r.number("scale"), window=mask.integer("size"), rot_base=rot.number("base"),
-                   rot_dims=rot.integer("dims"))
+        window, base, dims = None, 1.0, 0
+        if r.raw("mask") is not None:
+            window = JsonReader(_object(r.raw("mask"), where, "mask"), f"{where}.mask").integer("size")
+        if r.raw("rot") is not None:
+            rot = JsonReader(_object(r.raw("rot"), where, "rot"), f"{where}.rot")
+            base, dims = rot.number("base"), rot.integer("dims")
+        return cls(heads=r.integer("heads"), kv_heads=r.integer("kv_heads", r.integer("heads")), dim=dim,
+                   vdim=r.integer("vdim", dim), scale=r.number("scale"), window=window, rot_base=base, rot_dims=dims)
 
     def check(self, where: str) -> None:
-        require_positive(where, heads=self.heads, kv_heads=self.kv_heads, dim=self.dim, vdim=self.vdim,
-                         window=self.window, rot_dims=self.rot_dims)
+        require_positive(where, heads=self.heads, kv_heads=self.kv_heads, dim=self.dim, vdim=self.vdim)
+        if self.window is not None:
+            require_positive(where, window=self.window)
         if self.heads % self.kv_heads:
             raise ConfigError(f"'{where}': {self.heads} query heads cannot be shared out evenly over {self.kv_heads} "
                               "key/value heads")
-        if self.rot_dims % 2 or self.rot_dims > self.dim:
+        if self.rot_dims < 0 or self.rot_dims % 2 or self.rot_dims > self.dim:
             raise ConfigError(f"'{where}': rot.dims ({self.rot_dims}) must be even and at most dim ({self.dim})")
-        if not self.rot_base > 0:
+        if self.rot_dims and not self.rot_base > 0:
             raise ConfigError(f"'{where}': rot.base must be positive")
 
     def to_dict(self) -> Dict[str, Any]:
-        return {"dim": self.dim, "heads": self.heads, "kv_heads": self.kv_heads, "mask": {"size": self.window},
-                "rot": {"base": self.rot_base, "dims": self.rot_dims}, "scale": self.scale, "vdim": self.vdim}
+        out: Dict[str, Any] = {"dim": self.dim, "heads": self.heads, "kv_heads": self.kv_heads, "scale": self.scale,
+                               "vdim": self.vdim}
+        if self.window is not None:
+            out["mask"] = {"size": self.window}
+        if self.rot_dims:
+            out["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
+        return out
 
 
 @dataclass
@@ -281,9 +290,11 @@ class KesovikConfig(ModelConfig):
                 mixer = PartSpec("lightning", self._lightning_params(layer.lightning, "mix"))
             else:
                 left = layer.left
-                rope = f"rope:{left.rot_base!r}:{left.rot_dims}:{left.dim}"
-                positions.setdefault(rope, PartSpec("rope", {"theta": left.rot_base, "rotary_dim": left.rot_dims,
-                                                             "head_dim": left.dim, "pairing": "interleaved"}))
+                rope = None
+                if left.rot_dims:
+                    rope = f"rope:{left.rot_base!r}:{left.rot_dims}:{left.dim}"
+                    positions.setdefault(rope, PartSpec("rope", {"theta": left.rot_base, "rotary_dim": left.rot_dims,
+                                                                 "head_dim": left.dim, "pairing": "interleaved"}))
                 attention = {"hidden_size": self.width, "num_heads": left.heads, "num_kv_heads": left.kv_heads,
                              "head_dim": left.dim, "value_dim": left.vdim, "bias": True, "qk_norm": "projection",
                              "qk_norm_eps": self.norm_eps, "scale": left.scale, "window": left.window,

@@ -94,9 +94,11 @@ def window_attention(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: Dic
     q = (unit_rms(q, eps) * w[p + ".q.norm"]).view(t, heads, d)
     k = (unit_rms(k, eps) * w[p + ".k.norm"]).view(t, groups, d)
     positions = list(range(t))
-    q = rotate_pairs(q, positions, m["rot"]["base"], m["rot"]["dims"])
-    k = rotate_pairs(k, positions, m["rot"]["base"], m["rot"]["dims"])
-    o = window_scores_softmax(q, k, v.view(t, groups, dv), m["scale"], m["mask"]["size"])
+    if m.get("rot") is not None:                  # (a configuration that names no rotation has none)
+        q = rotate_pairs(q, positions, m["rot"]["base"], m["rot"]["dims"])
+        k = rotate_pairs(k, positions, m["rot"]["base"], m["rot"]["dims"])
+    window = m["mask"]["size"] if m.get("mask") is not None else t      # (and one that names no mask sees all before)
+    o = window_scores_softmax(q, k, v.view(t, groups, dv), m["scale"], window)
     return o.reshape(t, heads * dv) @ w[p + ".o"].T
 
 

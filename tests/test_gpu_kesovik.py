@@ -28,8 +28,12 @@ F64 = torch.float64
 
 
 def left(heads, kv_heads, dim, vdim, window, rot_dims, base, scale):
-    return {"dim": dim, "heads": heads, "kv_heads": kv_heads, "mask": {"size": window},
-            "rot": {"base": base, "dims": rot_dims}, "scale": scale, "vdim": vdim}
+    out = {"dim": dim, "heads": heads, "kv_heads": kv_heads, "scale": scale, "vdim": vdim}
+    if window is not None:
+        out["mask"] = {"size": window}
+    if rot_dims:
+        out["rot"] = {"base": base, "dims": rot_dims}
+    return out
 
 
 def lightning(heads, dim, vdim, decay):
@@ -124,9 +128,20 @@ def plain(folders):
 CLOSE_CALL = 0.006
 
 
-def agree(got, want, dtype, what, calls=(), first=0, tol=TOL):
+def agree(got, want, dtype, what, calls=(), first=0, tol=TOL, carried=False):
     """``close``; in bfloat16 without the positions at which a router's choice is a close call (``calls``, positions
-    in the sequence; row 0 of ``got`` is position ``first``), which must stay few."""
+    in the sequence; row 0 of ``got`` is position ``first``), which must stay few.  ``carried``: another choice at one
+    position may reach all later ones (through a state that forgets nothing, say) and close calls may be many: then
+    the positions before the first close call are compared one by one, and of the rest the median error."""
+    if dtype == "bfloat16" and calls and carried:
+        cut = max(0, min(calls) - first)
+        if cut:
+            close(got[:cut], want[:cut], dtype, what + " (before the first close call)", tol)
+        if cut < want.shape[0]:
+            rest = (got[cut:].double().cpu() - want[cut:].double().cpu()).abs().max(dim=1).values
+            assert torch.isfinite(rest).all(), what
+            assert float(rest.median()) <= tol[dtype] * max(1.0, float(want.abs().max())), f"{what}: median error {float(rest.median()):.3e}"
+        return
     if dtype == "bfloat16" and calls:
         keep = [i for i in range(want.shape[0]) if i + first not in calls]
         assert len(keep) >= 0.7 * want.shape[0] or want.shape[0] < 10, f"{what}: too many close calls to say anything"
@@ -674,8 +689,9 @@ def random_config(rng):
         if rng.random() < 0.6:
             groups, share = rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 4])
             dim = rng.choice([16, 24, 32, 48, 64])
-            rot = rng.choice([d for d in (2, 8, 16, 24, dim) if d <= dim])
-            mixer = parallel(left(groups * share, groups, dim, rng.choice([8, 16, 40, 48, 64]), rng.choice([1, 5, 16, 33, 100]),
+            rot = rng.choice([d for d in (0, 2, 8, 16, 24, dim) if d <= dim])      # (0: the configuration names no rotation)
+            mixer = parallel(left(groups * share, groups, dim, rng.choice([8, 16, 40, 48, 64]),
+                                  rng.choice([1, 5, 16, 33, 100, None]),
                                   rot, rng.choice([100.0, 1e4, 5e5]), rng.choice([0.1, dim ** -0.5, 0.5])),
                              light, rng.choice([0.5, 1.0, 1.5]), rng.choice([0.7, 1.0]))
         else:
@@ -694,7 +710,7 @@ def random_config(rng):
                   rng.choice([1.0, 3.0]), rng.choice([5.0, 15.0, 50.0]), layers)
 
 
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", range(12))
 def test_random_configurations(tmp_path, seed):
     """Whole, with the last 20 tokens one by one, and in portions of 2 to 70 tokens, in 32-bit and in bfloat16."""
     if not torch.cuda.is_available():
@@ -719,14 +735,14 @@ def test_random_configurations(tmp_path, seed):
         _, model = load_model(folder, mode=dtype)
         runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=4)
         whole = run_alone(runner, ids, [length])
-        agree(whole, want, dtype, f"whole: {what}", calls)
-        agree(run_alone(runner, ids, [length - 20] + [1] * 20), want, dtype, f"tail: {what}", calls)
+        agree(whole, want, dtype, f"whole: {what}", calls, carried=True)
+        agree(run_alone(runner, ids, [length - 20] + [1] * 20), want, dtype, f"tail: {what}", calls, carried=True)
         cuts, left_over, sizes = [], length, [40, 2, 17, 3, 70, 5, 19]
         while left_over:
             n = min(sizes[len(cuts) % len(sizes)], left_over)
             cuts.append(n)
             left_over -= n
-        agree(run_alone(runner, ids, cuts), want, dtype, f"portions {cuts}: {what}", calls)
+        agree(run_alone(runner, ids, cuts), want, dtype, f"portions {cuts}: {what}", calls, carried=True)
         del runner, model
     torch.cuda.empty_cache()
 

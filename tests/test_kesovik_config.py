@@ -53,7 +53,8 @@ def broken(path, value):
     (("layers", 0, "mixer", "left", "kv_heads"), 4),
     (("layers", 0, "mixer", "left", "rot", "dims"), 34),
     (("layers", 0, "mixer", "left", "rot", "dims"), 15),
-    (("layers", 0, "mixer", "left", "mask"), KeyError),
+    (("layers", 0, "mixer", "left", "mask", "size"), 0),
+    (("layers", 0, "mixer", "left", "scale"), KeyError),
     (("layers", 0, "mixer", "right", "decay"), [0.5, 0.9]),
     (("layers", 1, "mixer", "decay"), [0.5, 1.5]),
     (("layers", 1, "mixer", "dim"), 300),
@@ -79,6 +80,17 @@ def test_the_model_as_parts():
     assert branches[0]["params"]["window"] == 24 and branches[0]["params"]["value_dim"] == 16
     assert len(spec.positions) == 1 and next(iter(spec.positions.values())).params["rotary_dim"] == 16
     assert spec.embedding.params["scale"] == 2.0 and spec.head.params["softcap"] == 9.0
+
+
+def test_a_left_mixer_without_mask_or_rotation():
+    """What config.json does not name does not exist: no mask means every earlier token is visible, no rot no rotation."""
+    data = broken(("layers", 0, "mixer", "left", "mask"), KeyError)
+    del data["layers"][0]["mixer"]["left"]["rot"]
+    cfg = KesovikConfig.from_dict(data)
+    assert cfg.to_dict() == data
+    params = cfg.model_spec().layers[0].mixer.params["branches"][0]["params"]
+    assert params["window"] is None and params["position"] is None
+    assert not cfg.model_spec().positions
 
 
 def test_tensor_names_and_shapes():
